@@ -38,23 +38,44 @@ HIP_SOURCES = [
     "probe.hip",
 ]
 
+# Kernel groups that build into their own small library, so a process that
+# serves only one model family compiles (and loads) only what it runs.
+# libafmix.so: sequence-mixer op set (ops/seqmix.py).
+MIX_SOURCES = ["mix_glue.hip", "mix_seq.hip"]
+MIX_LIB = PKG_DIR / "libafmix.so"
 
-def _needs_build() -> bool:
-    if not LIB.exists():
+# hipcc -O3 may otherwise fuse scalar float code into packed-fp32 VALU ops
+HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _needs_build(lib: Path = LIB, sources=None) -> bool:
+    if not lib.exists():
         return True
-    lib_m = LIB.stat().st_mtime
-    deps = [CSRC / s for s in HIP_SOURCES] + [CSRC / "common.h", Path(__file__)]
+    lib_m = lib.stat().st_mtime
+    deps = [CSRC / s for s in (sources or HIP_SOURCES)] + \
+        [CSRC / "common.h", Path(__file__)]
     return any(d.stat().st_mtime > lib_m for d in deps)
+
+
+def build_mix(force: bool = False, verbose: bool = True) -> Path:
+    """Compile the sequence-mixer kernel group (libafmix.so) for gfx950."""
+    return _build_lib(MIX_LIB, MIX_SOURCES, force, verbose)
 
 
 def build_afops(force: bool = False, verbose: bool = True) -> Path:
     """Compile the HIP kernel library for gfx950 (incremental per-object)."""
-    if not force and not _needs_build():
-        return LIB
+    return _build_lib(LIB, HIP_SOURCES, force, verbose)
+
+
+def _build_lib(lib: Path, sources, force: bool, verbose: bool) -> Path:
+    if not force and not _needs_build(lib, sources):
+        return lib
+    import tempfile
     objdir = CSRC / ".obj"
     objdir.mkdir(exist_ok=True)
     objs = []
-    for src in HIP_SOURCES:
+    for src in sources:
         sp = CSRC / src
         op = objdir / (src + ".o")
         objs.append(op)
@@ -63,18 +84,28 @@ def build_afops(force: bool = False, verbose: bool = True) -> Path:
                 and op.stat().st_mtime > (CSRC / "common.h").stat().st_mtime):
             continue
         cmd = [
-            HIPCC, f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC",
-            "-fvisibility=hidden", "-c", str(sp), "-o", str(op),
+            HIPCC, f"--offload-arch={ARCH}", *HIP_FLAGS,
+            "-c", str(sp), "-o", str(op),
         ]
         if verbose:
             print("[afops]", " ".join(cmd), file=sys.stderr)
         subprocess.run(cmd, check=True)
+    # link to a temporary name and rename: a concurrent process never maps a
+    # half-written library
+    fd, tmp = tempfile.mkstemp(dir=str(lib.parent), prefix=lib.name + ".")
+    os.close(fd)
     cmd = [HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC",
-           *[str(o) for o in objs], "-o", str(LIB)]
+           *[str(o) for o in objs], "-o", tmp]
     if verbose:
         print("[afops]", " ".join(cmd), file=sys.stderr)
-    subprocess.run(cmd, check=True)
-    return LIB
+    try:
+        subprocess.run(cmd, check=True)
+        os.chmod(tmp, 0o755)
+        os.replace(tmp, lib)
+    finally:
+        if os.path.exists(tmp):
+            os.unlink(tmp)
+    return lib
 
 
 def build_native(force: bool = False, verbose: bool = True):
@@ -87,6 +118,7 @@ def build_native(force: bool = False, verbose: bool = True):
 
 def build_all(force: bool = False):
     build_afops(force=force)
+    build_mix(force=force)
     build_native(force=force)
 
 

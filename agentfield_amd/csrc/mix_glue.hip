@@ -1,0 +1,361 @@
+// Row-wise glue kernels of parallel-residual hybrid decoders: fp32 residual
+// stream, zero-centred RMSNorm pairs with token shift, per-head output norm
+// with SiLU gate, PolyNorm activation, sigmoid-gated residual add, softcap.
+//
+// Storage dtype S is bf16 (raw u16) or fp32; every statistic, gate and the
+// residual itself are fp32.  One workgroup (256 threads = 4 waves) per row
+// unless noted; rows are short (model width), so a row is read once into
+// registers/LDS-free strided loops and reduced with 64-wide wave shuffles.
+#include "common.h"
+
+namespace {
+
+template <typename S> __device__ __forceinline__ float ldf(const S* p);
+template <> __device__ __forceinline__ float ldf<u16>(const u16* p) { return bf2f(*p); }
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <typename S> __device__ __forceinline__ void stf(S* p, float v);
+template <> __device__ __forceinline__ void stf<u16>(u16* p, float v) { *p = f2bf(v); }
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+
+// Block-wide sum of up to N values per thread (256 threads); every thread
+// gets the totals.  red must hold N*4 floats.
+template <int N>
+__device__ __forceinline__ void block_sum(float (&v)[N], float* red) {
+#pragma unroll
+  for (int n = 0; n < N; ++n) v[n] = wave_sum_f32(v[n]);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();  // red may still be read from a previous call
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int n = 0; n < N; ++n) red[n * 4 + wave] = v[n];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int n = 0; n < N; ++n)
+    v[n] = red[n * 4] + red[n * 4 + 1] + red[n * 4 + 2] + red[n * 4 + 3];
+}
+
+template <typename S>
+__global__ void __launch_bounds__(256) embed_kernel(
+    float* __restrict__ out, const S* __restrict__ table,
+    const i32* __restrict__ ids, const float* __restrict__ add, int W) {
+  const int t = blockIdx.x;
+  const S* src = table + (size_t)ids[t] * W;
+  float* dst = out + (size_t)t * W;
+  for (int i = threadIdx.x; i < W; i += 256)
+    dst[i] = ldf<S>(src + i) + (add ? add[i] : 0.f);
+}
+
+__global__ void __launch_bounds__(256) add_rows_kernel(
+    float* __restrict__ x, const float* __restrict__ other,
+    const float* __restrict__ vec, i64 n, int W) {
+  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (i64)gridDim.x * 256) {
+    float v = x[i];
+    if (other) v += other[i];
+    if (vec) v += vec[i % W];
+    x[i] = v;
+  }
+}
+
+// a = norm(x)(1+w1), b = norm(x)(1+w2), s = a + (a_prev - a)*shift.
+template <typename S>
+__global__ void __launch_bounds__(256) dual_norm_shift_kernel(
+    S* __restrict__ a_out, S* __restrict__ s_out, S* __restrict__ b_out,
+    float* __restrict__ last, const float* __restrict__ x,
+    const S* __restrict__ w1, const S* __restrict__ w2,
+    const S* __restrict__ shift, const float* __restrict__ prev,
+    const i32* __restrict__ row_seq, const i32* __restrict__ cu,
+    const i32* __restrict__ q_start, const i32* __restrict__ sslot,
+    float eps, int W) {
+  __shared__ float red[8];
+  const int t = blockIdx.x;
+  const int b = row_seq[t];
+  const int r0 = cu[b];
+  const bool first = (t == r0);
+  const bool is_last = (t == cu[b + 1] - 1);
+  const int pos = q_start[b] + (t - r0);
+  const float* xr = x + (size_t)t * W;
+  const float* xp = xr - W;  // previous row, only touched when !first
+  const bool need_prev_row = shift && !first;
+  float ss[2] = {0.f, 0.f};
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const float v = xr[i];
+    ss[0] += v * v;
+    if (need_prev_row) {
+      const float p = xp[i];
+      ss[1] += p * p;
+    }
+  }
+  block_sum<2>(ss, red);
+  const float r = 1.0f / sqrtf(ss[0] / (float)W + eps);
+  const float rp = 1.0f / sqrtf(ss[1] / (float)W + eps);
+  const float* pv = (shift && first && pos > 0)
+                        ? prev + (size_t)sslot[b] * W : nullptr;
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const float xv = xr[i];
+    const float g1 = 1.0f + ldf<S>(w1 + i);
+    const float a = xv * r * g1;
+    stf<S>(a_out + (size_t)t * W + i, a);
+    if (b_out) stf<S>(b_out + (size_t)t * W + i, xv * r * (1.0f + ldf<S>(w2 + i)));
+    if (shift) {
+      float ap = 0.f;
+      if (need_prev_row) ap = xp[i] * rp * g1;
+      else if (pv) ap = pv[i];
+      stf<S>(s_out + (size_t)t * W + i, a + (ap - a) * ldf<S>(shift + i));
+      if (is_last) last[(size_t)b * W + i] = a;
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) scatter_state_kernel(
+    float* __restrict__ prev, const float* __restrict__ last,
+    const i32* __restrict__ sslot, const i32* __restrict__ cu, int W) {
+  const int b = blockIdx.x;
+  if (cu[b + 1] == cu[b]) return;
+  float* dst = prev + (size_t)sslot[b] * W;
+  const float* src = last + (size_t)b * W;
+  for (int i = threadIdx.x; i < W; i += 256) dst[i] = src[i];
+}
+
+template <typename S>
+__global__ void __launch_bounds__(256) norm_rows_kernel(
+    S* __restrict__ out, const float* __restrict__ x, const S* __restrict__ w,
+    const i32* __restrict__ rows, float eps, int W, int one_plus) {
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  const float* xr = x + (size_t)(rows ? rows[r] : r) * W;
+  float ss[1] = {0.f};
+  for (int i = threadIdx.x; i < W; i += 256) ss[0] += xr[i] * xr[i];
+  block_sum<1>(ss, red);
+  const float rs = 1.0f / sqrtf(ss[0] / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const float g = ldf<S>(w + i) + (one_plus ? 1.0f : 0.f);
+    stf<S>(out + (size_t)r * W + i, xr[i] * rs * g);
+  }
+}
+
+// One wave per (row, head): RMS over dv of fp32 o, * weight, * silu(gate).
+template <typename S>
+__global__ void __launch_bounds__(256) headnorm_gate_kernel(
+    S* __restrict__ out, const float* __restrict__ o, const S* __restrict__ g,
+    const S* __restrict__ w, float eps, int n_rh, int H, int dv, i64 ldg) {
+  const int rh = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (rh >= n_rh) return;
+  const int lane = threadIdx.x & 63;
+  const int t = rh / H, h = rh % H;
+  const float* orow = o + ((size_t)t * H + h) * dv;
+  float ss = 0.f;
+  for (int d = lane; d < dv; d += 64) ss += orow[d] * orow[d];
+  ss = wave_sum_f32(ss);
+  const float rs = 1.0f / sqrtf(ss / (float)dv + eps);
+  const S* grow = g + (size_t)t * ldg + (size_t)h * dv;
+  for (int d = lane; d < dv; d += 64) {
+    const float gv = ldf<S>(grow + d);
+    float v = orow[d] * rs;
+    if (w) v *= ldf<S>(w + d);
+    stf<S>(out + ((size_t)t * H + h) * dv + d, v * (gv / (1.0f + expf(-gv))));
+  }
+}
+
+template <typename S>
+__global__ void __launch_bounds__(256) polynorm_kernel(
+    S* __restrict__ out, const S* __restrict__ z, const float* __restrict__ coef,
+    float eps, int F, i64 ldz) {
+  __shared__ float red[12];
+  const int t = blockIdx.x;
+  const S* zr = z + (size_t)t * ldz;
+  float s[3] = {0.f, 0.f, 0.f};
+  for (int i = threadIdx.x; i < F; i += 256) {
+    const float v = ldf<S>(zr + i);
+    const float v2 = v * v;
+    s[0] += v2;
+    s[1] += v2 * v2;
+    s[2] += v2 * v2 * v2;
+  }
+  block_sum<3>(s, red);
+  const float r1 = 1.0f / sqrtf(s[0] / (float)F + eps);
+  const float r2 = 1.0f / sqrtf(s[1] / (float)F + eps);
+  const float r3 = 1.0f / sqrtf(s[2] / (float)F + eps);
+  const float c0 = coef[0], c1 = coef[1], c2 = coef[2], c3 = coef[3];
+  for (int i = threadIdx.x; i < F; i += 256) {
+    const float v = ldf<S>(zr + i);
+    const float v2 = v * v;
+    stf<S>(out + (size_t)t * F + i,
+           c0 * (v * r1) + c1 * (v2 * r2) + c2 * (v2 * v * r3) + c3);
+  }
+}
+
+template <typename S>
+__global__ void __launch_bounds__(256) gated_residual_kernel(
+    float* __restrict__ x, const S* __restrict__ a, float sa,
+    const S* __restrict__ b, float sb, const S* __restrict__ g1, i64 ldg1,
+    const float* __restrict__ b1, const S* __restrict__ m,
+    const S* __restrict__ g2, i64 ldg2, const float* __restrict__ b2,
+    int T, int W) {
+  const i64 n = (i64)T * W;
+  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (i64)gridDim.x * 256) {
+    const int t = (int)(i / W), c = (int)(i % W);
+    float mix = sa * ldf<S>(a + i);
+    if (b) mix += sb * ldf<S>(b + i);
+    const float z1 = ldf<S>(g1 + (size_t)t * ldg1 + c) + b1[c];
+    float add = mix / (1.0f + expf(-z1));
+    if (m) {
+      const float z2 = ldf<S>(g2 + (size_t)t * ldg2 + c) + b2[c];
+      add += ldf<S>(m + i) / (1.0f + expf(-z2));
+    }
+    x[i] += add;
+  }
+}
+
+template <typename S>
+__global__ void __launch_bounds__(256) softcap_kernel(
+    float* __restrict__ out, const S* __restrict__ in, float cap, i64 n) {
+  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (i64)gridDim.x * 256) {
+    const float v = ldf<S>(in + i);
+    out[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+  }
+}
+
+inline int grid_for(i64 n) {
+  i64 g = (n + 255) / 256;
+  return (int)(g < 1 ? 1 : (g > 8192 ? 8192 : g));
+}
+
+}  // namespace
+
+#define MIX_DISPATCH(dt, CALL_BF, CALL_F32) \
+  do {                                      \
+    if ((dt) == 0) { CALL_BF; }             \
+    else if ((dt) == 1) { CALL_F32; }       \
+    else return 9002;                       \
+  } while (0)
+
+AF_EXPORT int afm_embed(void* out, const void* table, const void* ids,
+                        const void* add, int T, int W, int dt, void* stream) {
+  if (T == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  MIX_DISPATCH(dt,
+      (embed_kernel<u16><<<T, 256, 0, s>>>((float*)out, (const u16*)table,
+          (const i32*)ids, (const float*)add, W)),
+      (embed_kernel<float><<<T, 256, 0, s>>>((float*)out, (const float*)table,
+          (const i32*)ids, (const float*)add, W)));
+  return af_last_err();
+}
+
+AF_EXPORT int afm_add_rows(void* x, const void* other, const void* vec, int T,
+                           int W, void* stream) {
+  if (T == 0) return 0;
+  const i64 n = (i64)T * W;
+  add_rows_kernel<<<grid_for(n), 256, 0, (hipStream_t)stream>>>(
+      (float*)x, (const float*)other, (const float*)vec, n, W);
+  return af_last_err();
+}
+
+AF_EXPORT int afm_dual_norm_shift(
+    void* a, void* s_out, void* b, void* last, const void* x, const void* w1,
+    const void* w2, const void* shift, const void* prev, const void* row_seq,
+    const void* cu, const void* q_start, const void* sslot, float eps, int T,
+    int W, int dt, void* stream) {
+  if (T == 0) return 0;
+  if (shift && (!prev || !last)) return 9003;
+  if ((b == nullptr) != (w2 == nullptr)) return 9003;
+  hipStream_t s = (hipStream_t)stream;
+  MIX_DISPATCH(dt,
+      (dual_norm_shift_kernel<u16><<<T, 256, 0, s>>>((u16*)a, (u16*)s_out,
+          (u16*)b, (float*)last, (const float*)x, (const u16*)w1,
+          (const u16*)w2, (const u16*)shift, (const float*)prev,
+          (const i32*)row_seq, (const i32*)cu, (const i32*)q_start,
+          (const i32*)sslot, eps, W)),
+      (dual_norm_shift_kernel<float><<<T, 256, 0, s>>>((float*)a,
+          (float*)s_out, (float*)b, (float*)last, (const float*)x,
+          (const float*)w1, (const float*)w2, (const float*)shift,
+          (const float*)prev, (const i32*)row_seq, (const i32*)cu,
+          (const i32*)q_start, (const i32*)sslot, eps, W)));
+  return af_last_err();
+}
+
+AF_EXPORT int afm_scatter_state(void* prev, const void* last,
+                                const void* sslot, const void* cu, int B,
+                                int W, void* stream) {
+  if (B == 0) return 0;
+  scatter_state_kernel<<<B, 256, 0, (hipStream_t)stream>>>(
+      (float*)prev, (const float*)last, (const i32*)sslot, (const i32*)cu, W);
+  return af_last_err();
+}
+
+AF_EXPORT int afm_norm_rows(void* out, const void* x, const void* w,
+                            const void* rows, float eps, int R, int W,
+                            int one_plus, int dt, void* stream) {
+  if (R == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  MIX_DISPATCH(dt,
+      (norm_rows_kernel<u16><<<R, 256, 0, s>>>((u16*)out, (const float*)x,
+          (const u16*)w, (const i32*)rows, eps, W, one_plus)),
+      (norm_rows_kernel<float><<<R, 256, 0, s>>>((float*)out, (const float*)x,
+          (const float*)w, (const i32*)rows, eps, W, one_plus)));
+  return af_last_err();
+}
+
+AF_EXPORT int afm_headnorm_gate(void* out, const void* o, const void* g,
+                                const void* w, float eps, int T, int H, int dv,
+                                i64 ldg, int dt, void* stream) {
+  if (T == 0) return 0;
+  const int n_rh = T * H;
+  const int grid = (n_rh + 3) / 4;
+  hipStream_t s = (hipStream_t)stream;
+  MIX_DISPATCH(dt,
+      (headnorm_gate_kernel<u16><<<grid, 256, 0, s>>>((u16*)out,
+          (const float*)o, (const u16*)g, (const u16*)w, eps, n_rh, H, dv, ldg)),
+      (headnorm_gate_kernel<float><<<grid, 256, 0, s>>>((float*)out,
+          (const float*)o, (const float*)g, (const float*)w, eps, n_rh, H, dv,
+          ldg)));
+  return af_last_err();
+}
+
+AF_EXPORT int afm_polynorm(void* out, const void* z, const void* coef,
+                           float eps, int T, int F, i64 ldz, int dt,
+                           void* stream) {
+  if (T == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  MIX_DISPATCH(dt,
+      (polynorm_kernel<u16><<<T, 256, 0, s>>>((u16*)out, (const u16*)z,
+          (const float*)coef, eps, F, ldz)),
+      (polynorm_kernel<float><<<T, 256, 0, s>>>((float*)out, (const float*)z,
+          (const float*)coef, eps, F, ldz)));
+  return af_last_err();
+}
+
+AF_EXPORT int afm_gated_residual(
+    void* x, const void* a, float sa, const void* b, float sb, const void* g1,
+    i64 ldg1, const void* b1, const void* m, const void* g2, i64 ldg2,
+    const void* b2, int T, int W, int dt, void* stream) {
+  if (T == 0) return 0;
+  if (m && (!g2 || !b2)) return 9003;
+  hipStream_t s = (hipStream_t)stream;
+  const int grid = grid_for((i64)T * W);
+  MIX_DISPATCH(dt,
+      (gated_residual_kernel<u16><<<grid, 256, 0, s>>>((float*)x,
+          (const u16*)a, sa, (const u16*)b, sb, (const u16*)g1, ldg1,
+          (const float*)b1, (const u16*)m, (const u16*)g2, ldg2,
+          (const float*)b2, T, W)),
+      (gated_residual_kernel<float><<<grid, 256, 0, s>>>((float*)x,
+          (const float*)a, sa, (const float*)b, sb, (const float*)g1, ldg1,
+          (const float*)b1, (const float*)m, (const float*)g2, ldg2,
+          (const float*)b2, T, W)));
+  return af_last_err();
+}
+
+AF_EXPORT int afm_softcap(void* out, const void* in, float cap, i64 n, int dt,
+                          void* stream) {
+  if (n == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  MIX_DISPATCH(dt,
+      (softcap_kernel<u16><<<grid_for(n), 256, 0, s>>>((float*)out,
+          (const u16*)in, cap, n)),
+      (softcap_kernel<float><<<grid_for(n), 256, 0, s>>>((float*)out,
+          (const float*)in, cap, n)));
+  return af_last_err();
+}

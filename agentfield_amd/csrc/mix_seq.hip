@@ -1,0 +1,356 @@
+// Sequence mixers over packed row chunks: whole-row q/k RMSNorm + paged
+// cache append, masked (causal / chunk-local / banded) paged softmax
+// attention for arbitrary head sizes, and the token-serial decayed
+// outer-product recurrence with per-sequence fp32 state slots.
+//
+// Storage dtype S is bf16 (raw u16) or fp32; scores, softmax, decays and the
+// recurrent state are fp32.
+#include "common.h"
+
+namespace {
+
+template <typename S> __device__ __forceinline__ float ldf(const S* p);
+template <> __device__ __forceinline__ float ldf<u16>(const u16* p) { return bf2f(*p); }
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <typename S> __device__ __forceinline__ void stf(S* p, float v);
+template <> __device__ __forceinline__ void stf<u16>(u16* p, float v) { *p = f2bf(v); }
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+
+// ---------------------------------------------------------------- qk norm
+// One workgroup per row.  q row [nq], k row [nk], v row [nv]; caches
+// [P, G, page, dk|dv]; slot = page_index*page + offset.
+template <typename S>
+__global__ void __launch_bounds__(256) qk_norm_cache_kernel(
+    S* __restrict__ qout, const S* __restrict__ q, const S* __restrict__ k,
+    const S* __restrict__ v, const S* __restrict__ qw, const S* __restrict__ kw,
+    S* __restrict__ kc, S* __restrict__ vc, const i64* __restrict__ slots,
+    float eps, int nq, int nk, int nv, int G, int dk, int dv, int page,
+    i64 ldq, i64 ldk, i64 ldv) {
+  __shared__ float red[8];
+  const int t = blockIdx.x;
+  const S* qr = q + (size_t)t * ldq;
+  const S* kr = k + (size_t)t * ldk;
+  const S* vr = v + (size_t)t * ldv;
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x; i < nq; i += 256) { const float f = ldf<S>(qr + i); sq += f * f; }
+  for (int i = threadIdx.x; i < nk; i += 256) { const float f = ldf<S>(kr + i); sk += f * f; }
+  sq = wave_sum_f32(sq);
+  sk = wave_sum_f32(sk);
+  if ((threadIdx.x & 63) == 0) {
+    red[threadIdx.x >> 6] = sq;
+    red[4 + (threadIdx.x >> 6)] = sk;
+  }
+  __syncthreads();
+  const float rq = qw ? 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)nq + eps) : 1.0f;
+  const float rk = kw ? 1.0f / sqrtf((red[4] + red[5] + red[6] + red[7]) / (float)nk + eps) : 1.0f;
+  for (int i = threadIdx.x; i < nq; i += 256) {
+    float f = ldf<S>(qr + i) * rq;
+    if (qw) f *= ldf<S>(qw + i);
+    stf<S>(qout + (size_t)t * nq + i, f);
+  }
+  const i64 sl = slots[t];
+  if (sl < 0) return;
+  const i64 pg = sl / page, off = sl % page;
+  for (int i = threadIdx.x; i < nk; i += 256) {
+    const int g = i / dk, d = i % dk;
+    float f = ldf<S>(kr + i) * rk;
+    if (kw) f *= ldf<S>(kw + i);
+    stf<S>(kc + (((size_t)pg * G + g) * page + off) * dk + d, f);
+  }
+  for (int i = threadIdx.x; i < nv; i += 256) {
+    const int g = i / dv, d = i % dv;
+    vc[(((size_t)pg * G + g) * page + off) * dv + d] = vr[i];
+  }
+}
+
+// -------------------------------------------------------- masked attention
+// One wave per (row, query head), 4 waves per workgroup.  Keys are walked in
+// tiles of 64 (one key per lane for the scores, one output channel per lane
+// for P.V), online softmax across tiles.  MAXV = ceil(dv/64) accumulators.
+template <typename S, int MAXV>
+__global__ void __launch_bounds__(256) masked_attention_kernel(
+    S* __restrict__ out, const S* __restrict__ q, const S* __restrict__ kc,
+    const S* __restrict__ vc, const i32* __restrict__ bt,
+    const i32* __restrict__ row_seq, const i32* __restrict__ positions,
+    float scale, int n_rh, int H, int G, int dk, int dv, int page, int maxp,
+    int chunk, int window, i64 ldq) {
+  extern __shared__ float smem[];           // [4][dk + 64]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int rh = blockIdx.x * 4 + wave;
+  if (rh >= n_rh) return;                    // whole wave exits together
+  float* qs = smem + wave * (dk + 64);
+  float* ps = qs + dk;
+  const int t = rh / H, h = rh % H;
+  const int g = h / (H / G);
+  const int pos = positions[t];
+  const i32* btr = bt + (size_t)row_seq[t] * maxp;
+  int lo = 0;
+  if (chunk > 0) lo = (pos / chunk) * chunk;
+  if (window > 0 && pos - window + 1 > lo) lo = pos - window + 1;
+  const S* qr = q + (size_t)t * ldq + (size_t)h * dk;
+  for (int d = lane; d < dk; d += 64) qs[d] = ldf<S>(qr + d) * scale;
+  float m = AF_NEG_INF, l = 0.f;
+  float acc[MAXV];
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) acc[i] = 0.f;
+  for (int j0 = lo; j0 <= pos; j0 += 64) {
+    const int j = j0 + lane;
+    float s = AF_NEG_INF;
+    if (j <= pos) {
+      const int pg = btr[j / page];
+      const S* kr = kc + (((size_t)pg * G + g) * page + (j % page)) * dk;
+      float d0 = 0.f;
+      for (int d = 0; d < dk; ++d) d0 += qs[d] * ldf<S>(kr + d);
+      s = d0;
+    }
+    const float mn = fmaxf(m, wave_max_f32(s));
+    const float corr = expf(m - mn);
+    const float p = (j <= pos) ? expf(s - mn) : 0.f;
+    l = l * corr + wave_sum_f32(p);
+    m = mn;
+    __builtin_amdgcn_wave_barrier();
+    ps[lane] = p;                            // wave-private LDS: ordered without a block barrier
+    __builtin_amdgcn_wave_barrier();
+    const int cnt = min(64, pos - j0 + 1);
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+      const int d = lane + 64 * i;
+      float a = acc[i] * corr;
+      if (d < dv) {
+        for (int jj = 0; jj < cnt; ++jj) {
+          const int jk = j0 + jj;
+          const int pg = btr[jk / page];
+          a += ps[jj] * ldf<S>(vc + (((size_t)pg * G + g) * page + (jk % page)) * dv + d);
+        }
+      }
+      acc[i] = a;
+    }
+  }
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int d = lane + 64 * i;
+    if (d < dv) stf<S>(out + ((size_t)t * H + h) * dv + d, acc[i] * inv);
+  }
+}
+
+// ------------------------------------------------------------- linear scan
+// Workgroup = (sequence, head, 32-column tile of dv); 256 threads = 8 row
+// groups x 32 columns.  Thread (r, c) keeps rows r, r+8, ... of column c of
+// the state in registers (RP rows).  Tokens are walked serially; q/k/decay
+// rows are staged through double-buffered LDS (rotary + scaling applied on
+// the way in), partial outputs are reduced across the 8 row groups through a
+// double-buffered LDS tile one token late, so a token costs one barrier.
+template <typename S, int RP>
+__global__ void __launch_bounds__(256) linear_scan_kernel(
+    float* __restrict__ out, float* __restrict__ state,
+    const S* __restrict__ q, const S* __restrict__ k, const S* __restrict__ v,
+    const S* __restrict__ zl, const float* __restrict__ zbias,
+    const float* __restrict__ head_decay, const float* __restrict__ inv_freq,
+    const i32* __restrict__ positions, const i32* __restrict__ cu,
+    const i32* __restrict__ q_start, const i32* __restrict__ sslot,
+    float q_scale, float k_scale, float inv_tau, int H, int dk, int dv,
+    int rot, i64 ldq, i64 ldk, i64 ldv, i64 ldz) {
+  extern __shared__ float smem[];  // [2][3*dk] + [2][8*32]
+  const int b = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 32;
+  const int t0 = cu[b], t1 = cu[b + 1];
+  if (t1 <= t0) return;
+  const int r = threadIdx.x >> 5, cc = threadIdx.x & 31;
+  const int c = c0 + cc;
+  const bool cok = c < dv;
+  float* stage = smem;                 // [2][3][dk]: q, k, decay
+  float* red = smem + 6 * dk;          // [2][8][32]
+  float* sbase = state + (((size_t)sslot[b] * H + h) * dk) * dv;
+  float st[RP];
+  const bool fresh = q_start[b] == 0;
+#pragma unroll
+  for (int ii = 0; ii < RP; ++ii) {
+    const int i = r + 8 * ii;
+    st[ii] = (!fresh && cok && i < dk) ? sbase[(size_t)i * dv + c] : 0.f;
+  }
+  const float hd = head_decay ? head_decay[h] : 1.0f;
+  const int half = rot >> 1;
+  for (int t = t0; t < t1; ++t) {
+    float* sq = stage + (size_t)((t - t0) & 1) * 3 * dk;
+    float* sk = sq + dk;
+    float* sa = sk + dk;
+    const S* qr = q + (size_t)t * ldq + (size_t)h * dk;
+    const S* kr = k + (size_t)t * ldk + (size_t)h * dk;
+    const float posf = (float)positions[t];
+    for (int i = threadIdx.x; i < dk; i += 256) {
+      float qv = ldf<S>(qr + i), kv = ldf<S>(kr + i);
+      if (i < rot) {
+        const bool lowh = i < half;
+        const int fi = lowh ? i : i - half;
+        const int pi = lowh ? i + half : i - half;
+        const float ang = posf * inv_freq[fi];
+        const float cs = cosf(ang), sn = sinf(ang);
+        const float qp = ldf<S>(qr + pi), kp = ldf<S>(kr + pi);
+        // pair (u, w) -> (u cos - w sin, w cos + u sin)
+        qv = lowh ? qv * cs - qp * sn : qv * cs + qp * sn;
+        kv = lowh ? kv * cs - kp * sn : kv * cs + kp * sn;
+      }
+      sq[i] = qv * q_scale;
+      sk[i] = kv * k_scale;
+      float a = hd;
+      if (zl) {
+        const float z = ldf<S>(zl + (size_t)t * ldz + (size_t)h * dk + i) + zbias[(size_t)h * dk + i];
+        // log(sigmoid(z)) = -softplus(-z), evaluated without overflow
+        const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
+        a = expf(ls * inv_tau);
+      }
+      sa[i] = a;
+    }
+    const float vv = cok ? ldf<S>(v + (size_t)t * ldv + (size_t)h * dv + c) : 0.f;
+    __syncthreads();
+    if (t > t0 && r == 0 && cok) {
+      const float* rd = red + (size_t)((t - 1 - t0) & 1) * 256;
+      float o = 0.f;
+#pragma unroll
+      for (int rr = 0; rr < 8; ++rr) o += rd[rr * 32 + cc];
+      out[(size_t)(t - 1) * H * dv + (size_t)h * dv + c] = o;
+    }
+    float part = 0.f;
+#pragma unroll
+    for (int ii = 0; ii < RP; ++ii) {
+      const int i = r + 8 * ii;
+      if (i < dk) {
+        st[ii] = sa[i] * st[ii] + sk[i] * vv;
+        part += st[ii] * sq[i];
+      }
+    }
+    red[(size_t)((t - t0) & 1) * 256 + r * 32 + cc] = part;
+  }
+  __syncthreads();
+  if (r == 0 && cok) {
+    const float* rd = red + (size_t)((t1 - 1 - t0) & 1) * 256;
+    float o = 0.f;
+#pragma unroll
+    for (int rr = 0; rr < 8; ++rr) o += rd[rr * 32 + cc];
+    out[(size_t)(t1 - 1) * H * dv + (size_t)h * dv + c] = o;
+  }
+  if (cok) {
+#pragma unroll
+    for (int ii = 0; ii < RP; ++ii) {
+      const int i = r + 8 * ii;
+      if (i < dk) sbase[(size_t)i * dv + c] = st[ii];
+    }
+  }
+}
+
+}  // namespace
+
+AF_EXPORT int afm_qk_norm_cache(
+    void* qout, const void* q, const void* k, const void* v, const void* qw,
+    const void* kw, void* kc, void* vc, const void* slots, float eps, int T,
+    int nq, int nk, int nv, int G, int dk, int dv, int page, i64 ldq, i64 ldk,
+    i64 ldv, int dt, void* stream) {
+  if (T == 0) return 0;
+  if (nk != G * dk || nv != G * dv) return 9003;
+  hipStream_t s = (hipStream_t)stream;
+  if (dt == 0)
+    qk_norm_cache_kernel<u16><<<T, 256, 0, s>>>((u16*)qout, (const u16*)q,
+        (const u16*)k, (const u16*)v, (const u16*)qw, (const u16*)kw, (u16*)kc,
+        (u16*)vc, (const i64*)slots, eps, nq, nk, nv, G, dk, dv, page, ldq,
+        ldk, ldv);
+  else if (dt == 1)
+    qk_norm_cache_kernel<float><<<T, 256, 0, s>>>((float*)qout,
+        (const float*)q, (const float*)k, (const float*)v, (const float*)qw,
+        (const float*)kw, (float*)kc, (float*)vc, (const i64*)slots, eps, nq,
+        nk, nv, G, dk, dv, page, ldq, ldk, ldv);
+  else
+    return 9002;
+  return af_last_err();
+}
+
+template <typename S>
+static int launch_attention(void* out, const void* q, const void* kc,
+                            const void* vc, const void* bt, const void* row_seq,
+                            const void* positions, float scale, int T, int H,
+                            int G, int dk, int dv, int page, int maxp,
+                            int chunk, int window, i64 ldq, hipStream_t s) {
+  const int n_rh = T * H;
+  const int grid = (n_rh + 3) / 4;
+  const size_t sm = (size_t)4 * (dk + 64) * sizeof(float);
+#define ATT(MV)                                                              \
+  masked_attention_kernel<S, MV><<<grid, 256, sm, s>>>(                      \
+      (S*)out, (const S*)q, (const S*)kc, (const S*)vc, (const i32*)bt,      \
+      (const i32*)row_seq, (const i32*)positions, scale, n_rh, H, G, dk, dv, \
+      page, maxp, chunk, window, ldq)
+  if (dv <= 64) ATT(1);
+  else if (dv <= 128) ATT(2);
+  else ATT(4);
+#undef ATT
+  return af_last_err();
+}
+
+AF_EXPORT int afm_masked_attention(
+    void* out, const void* q, const void* kc, const void* vc, const void* bt,
+    const void* row_seq, const void* positions, float scale, int T, int H,
+    int G, int dk, int dv, int page, int maxp, int chunk, int window, i64 ldq,
+    int dt, void* stream) {
+  if (T == 0) return 0;
+  if (G <= 0 || H % G || dv > 256 || dk > 1024) return 9003;
+  hipStream_t s = (hipStream_t)stream;
+  if (dt == 0)
+    return launch_attention<u16>(out, q, kc, vc, bt, row_seq, positions, scale,
+                                 T, H, G, dk, dv, page, maxp, chunk, window,
+                                 ldq, s);
+  if (dt == 1)
+    return launch_attention<float>(out, q, kc, vc, bt, row_seq, positions,
+                                   scale, T, H, G, dk, dv, page, maxp, chunk,
+                                   window, ldq, s);
+  return 9002;
+}
+
+template <typename S>
+static int launch_scan(float* out, float* state, const void* q, const void* k,
+                       const void* v, const void* zl, const float* zbias,
+                       const float* head_decay, const float* inv_freq,
+                       const i32* positions, const i32* cu, const i32* q_start,
+                       const i32* sslot, float q_scale, float k_scale,
+                       float inv_tau, int B, int H, int dk, int dv, int rot,
+                       i64 ldq, i64 ldk, i64 ldv, i64 ldz, hipStream_t s) {
+  dim3 grid(B, H, (dv + 31) / 32);
+  const size_t sm = (size_t)(6 * dk + 512) * sizeof(float);
+  const int rp = (dk + 7) / 8;
+#define SCAN(RP)                                                             \
+  linear_scan_kernel<S, RP><<<grid, 256, sm, s>>>(                           \
+      out, state, (const S*)q, (const S*)k, (const S*)v, (const S*)zl, zbias, \
+      head_decay, inv_freq, positions, cu, q_start, sslot, q_scale, k_scale, \
+      inv_tau, H, dk, dv, rot, ldq, ldk, ldv, ldz)
+  if (rp <= 4) SCAN(4);
+  else if (rp <= 8) SCAN(8);
+  else if (rp <= 16) SCAN(16);
+  else SCAN(32);
+#undef SCAN
+  return af_last_err();
+}
+
+AF_EXPORT int afm_linear_scan(
+    void* out, void* state, const void* q, const void* k, const void* v,
+    const void* zl, const void* zbias, const void* head_decay,
+    const void* inv_freq, const void* positions, const void* cu,
+    const void* q_start, const void* sslot, float q_scale, float k_scale,
+    float inv_tau, int B, int H, int dk, int dv, int rot, i64 ldq, i64 ldk,
+    i64 ldv, i64 ldz, int dt, void* stream) {
+  if (B == 0) return 0;
+  if (dk > 256 || dk < 1 || dv < 1) return 9003;
+  if (rot < 0 || rot > dk || (rot & 1) || (rot && !inv_freq)) return 9003;
+  if ((zl == nullptr) == (head_decay == nullptr)) return 9003;
+  if (zl && !zbias) return 9003;
+  hipStream_t s = (hipStream_t)stream;
+  if (dt == 0)
+    return launch_scan<u16>((float*)out, (float*)state, q, k, v, zl,
+        (const float*)zbias, (const float*)head_decay, (const float*)inv_freq,
+        (const i32*)positions, (const i32*)cu, (const i32*)q_start,
+        (const i32*)sslot, q_scale, k_scale, inv_tau, B, H, dk, dv, rot, ldq,
+        ldk, ldv, ldz, s);
+  if (dt == 1)
+    return launch_scan<float>((float*)out, (float*)state, q, k, v, zl,
+        (const float*)zbias, (const float*)head_decay, (const float*)inv_freq,
+        (const i32*)positions, (const i32*)cu, (const i32*)q_start,
+        (const i32*)sslot, q_scale, k_scale, inv_tau, B, H, dk, dv, rot, ldq,
+        ldk, ldv, ldz, s);
+  return 9002;
+}

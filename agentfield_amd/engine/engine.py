@@ -1,4 +1,5 @@
-"""The serving engine: continuous batching over the paged-KV Llama model.
+"""The serving engine: continuous batching over a paged-KV decoder (Llama
+family) or a paged-KV + state-slot decoder (hybrid families).
 
 One engine instance drives one GPU (DP replica) or one TP rank group.
 Decode steps are hipGraph-captured per batch-size bucket: the whole
@@ -15,7 +16,8 @@ import torch
 from .. import ops
 from ..models.llama import (AttnMetadata, KVCache, LlamaConfig,
                             LlamaForCausalLM)
-from .scheduler import ScheduleBatch, SchedulerConfig, make_scheduler
+from .scheduler import (ScheduleBatch, SchedulerConfig, SlotAllocator,
+                        make_scheduler)
 from .sequence import SamplingParams, Sequence, SeqStatus
 
 DECODE_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
@@ -47,16 +49,32 @@ class LLMEngine:
                  tp_group=None, spec_lookup: int = 0,
                  spec_draft=None, spec_draft_k: int = 4,
                  draft_model: "LlamaForCausalLM | None" = None,
-                 prefix_cache: bool = False):
+                 prefix_cache: bool = False, caller_paced: bool = False):
         self.cfg = cfg
         self.device = torch.device(device)
         self.is_gpu = self.device.type == "cuda"
         self.tp_group = tp_group
         if model is None:
-            model = LlamaForCausalLM(cfg, device=device, dtype=dtype).init_random(seed)
+            from ..models.registry import build_model
+            model = build_model(cfg, device=device,
+                                dtype=dtype).init_random(seed)
         self.model = model.eval()
+        # models with per-sequence state besides K/V get a slot per running
+        # sequence (slot 0 = null lane), handed out next to the pages
+        self.stateful = bool(getattr(model, "needs_state_slots", False))
+        if self.stateful:
+            if (spec_lookup or spec_draft is not None
+                    or draft_model is not None) and \
+                    not getattr(model, "supports_speculation", False):
+                raise ValueError("speculative decoding needs state rollback, "
+                                 "which this model family does not provide")
+            if prefix_cache and not getattr(model, "supports_prefix_cache",
+                                            False):
+                raise ValueError("prefix caching cannot restore recurrent "
+                                 "state; not available for this model family")
         if self.device.type == "cuda" and tp_group is None and \
-                not getattr(model, "no_fused_decode", False):
+                not getattr(model, "no_fused_decode", False) and \
+                hasattr(self.model, "fold_norm_weights"):
             self.model.fold_norm_weights()
 
         if num_pages is None:
@@ -65,10 +83,20 @@ class LLMEngine:
                 budget = int(free * kv_memory_frac)
             else:
                 budget = 64 << 20
-            num_pages = max(16, budget // KVCache.bytes_per_page(cfg, page_size))
+            per_page = (self.model.cache_bytes_per_page(page_size)
+                        if hasattr(self.model, "cache_bytes_per_page")
+                        else KVCache.bytes_per_page(cfg, page_size))
+            num_pages = max(16, budget // per_page)
         max_pages_per_seq = (cfg.max_position + page_size - 1) // page_size
         self.max_pages_per_seq = max_pages_per_seq
-        self.kv = KVCache(cfg, num_pages, page_size, self.device, dtype)
+        if hasattr(self.model, "make_cache"):
+            self.kv = self.model.make_cache(num_pages, page_size,
+                                            max_num_seqs + 1, self.device,
+                                            dtype)
+        else:
+            self.kv = KVCache(cfg, num_pages, page_size, self.device, dtype)
+        self.state_slots = SlotAllocator(max_num_seqs) if self.stateful \
+            else None
         # draft-model speculation (greedy-exact): a small model proposes
         # spec_draft_k tokens per step; the main model verifies them in
         # one chunked forward (_step_verify — shared with prompt-lookup).
@@ -125,12 +153,16 @@ class LLMEngine:
                 from .prefix_cache import PrefixCachingScheduler
                 self.sched = PrefixCachingScheduler(sched_cfg)
         else:
-            self.sched = make_scheduler(sched_cfg)
+            # caller-paced requests reserve pages token by token, which the
+            # Python scheduler implements
+            self.sched = make_scheduler(sched_cfg,
+                                        prefer_native=not caller_paced)
         self.page_size = page_size
         self.eos_id = eos_id
         self.max_num_seqs = max_num_seqs
         self._next_id = 0
         self._prefilling: list[Sequence] = []
+        self._open: dict[int, Sequence] = {}   # caller-paced requests
         self._finished: dict[int, Sequence] = {}
         self.sampler = ops.SamplerState(max_num_seqs, self.device, seed=seed or 0x5EED)
         # MoE decode graph-captures too: the static-capacity dispatch
@@ -183,6 +215,11 @@ class LLMEngine:
             "topk": torch.zeros(B, dtype=torch.int32, device=dev),
             "topp": torch.ones(B, dtype=torch.float32, device=dev),
             "tokens": torch.zeros(B, dtype=torch.int32, device=dev),
+            # stateful models: slot per lane + the packed-chunk view of a
+            # decode step (one row per sequence)
+            "sslot": torch.zeros(B, dtype=torch.int32, device=dev),
+            "cu": torch.arange(B + 1, dtype=torch.int32, device=dev),
+            "rowseq": torch.arange(B, dtype=torch.int32, device=dev),
             # logprob reporting (filled only in lp-keyed graphs)
             "lp_tok": torch.zeros(B, dtype=torch.float32, device=dev),
             "lp_vals": torch.zeros(B, LP_TOPN, dtype=torch.float32, device=dev),
@@ -190,7 +227,8 @@ class LLMEngine:
         }
         self._host = {k: torch.zeros_like(v, device="cpu").pin_memory()
                       if self.is_gpu else torch.zeros_like(v)
-                      for k, v in self._dec.items()}
+                      for k, v in self._dec.items()
+                      if k not in ("cu", "rowseq")}
         # block-table dirty tracking: row -> (seq_id, pages_written)
         self._bt_rows: dict[int, tuple] = {}
 
@@ -232,6 +270,8 @@ class LLMEngine:
             elif seq in self.sched.waiting:
                 self.sched.waiting.remove(seq)
             self.sched.release(seq)
+        if self.state_slots is not None:
+            self.state_slots.release(seq)
         seq.status = SeqStatus.FINISHED
         seq.finish_reason = "cancelled"
         self._finished[seq_id] = seq
@@ -293,6 +333,8 @@ class LLMEngine:
             if done:
                 seq.finish_ns = now
                 self.sched.finish(seq)
+                if self.state_slots is not None:
+                    self.state_slots.release(seq)
                 self._finished[seq.seq_id] = seq
             if self._emit(seq, done):
                 if seq.on_token is not None:
@@ -316,6 +358,104 @@ class LLMEngine:
         return seq.pages[tok_idx // self.page_size] * self.page_size + \
             tok_idx % self.page_size
 
+    def _state_slot(self, seq: Sequence) -> int:
+        live = None
+        if self.state_slots.num_free == 0:
+            running = getattr(self.sched, "running", None)
+            if running is not None:
+                live = {s.seq_id for s in running}
+                live.update(s.seq_id for s in self._prefilling)
+                live.update(self._open)
+        return self.state_slots.slot_of(seq, live)
+
+    def _chunk_batch(self, seqs: list[Sequence], starts: list[int],
+                     token_lists: list[list[int]]):
+        """Device-side description of one packed step: sequence i runs
+        token_lists[i] at absolute positions starts[i].. — prompt portions
+        and single decoded tokens alike.  Returns (ids, positions, metadata,
+        row offsets)."""
+        dev = self.device
+        ids, pos, slots, rowseq, bt_rows = [], [], [], [], []
+        for i, (seq, np0, toks) in enumerate(zip(seqs, starts, token_lists)):
+            take = len(toks)
+            ids.extend(toks)
+            pos.extend(range(np0, np0 + take))
+            slots.extend(self._slot(seq, j) for j in range(np0, np0 + take))
+            rowseq.extend([i] * take)
+            row = torch.zeros(self.max_pages_per_seq, dtype=torch.int32)
+            row[:len(seq.pages)] = torch.tensor(seq.pages, dtype=torch.int32)
+            bt_rows.append(row)
+        chunks = [len(t) for t in token_lists]
+        cu_list = [0]
+        for ln in chunks:
+            cu_list.append(cu_list[-1] + ln)
+        md = AttnMetadata(
+            is_prefill=True,
+            slots=torch.tensor(slots, dtype=torch.int64, device=dev),
+            cu_seqlens=torch.tensor(cu_list, dtype=torch.int32, device=dev),
+            seq_lens=chunks,
+            q_start=torch.tensor(starts, dtype=torch.int32, device=dev),
+            block_table=torch.stack(bt_rows).to(dev))
+        if self.stateful:
+            md.state_slots = torch.tensor(
+                [self._state_slot(s) for s in seqs], dtype=torch.int32,
+                device=dev)
+            md.row_seq = torch.tensor(rowseq, dtype=torch.int32, device=dev)
+        return (torch.tensor(ids, dtype=torch.int32, device=dev),
+                torch.tensor(pos, dtype=torch.int32, device=dev), md, cu_list)
+
+    # -- caller-paced requests: tokens are given, logits are returned -------
+    def open_request(self) -> Sequence:
+        """Admit a request whose tokens the caller supplies step by step
+        (feed_step); it holds pages and a state slot until close_request."""
+        if not hasattr(self.sched, "admit_open"):
+            raise RuntimeError("caller-paced requests need "
+                               "LLMEngine(caller_paced=True)")
+        if len(self._open) >= self.max_num_seqs:
+            raise MemoryError("more open requests than max_num_seqs")
+        seq = Sequence(self._next_id, [], SamplingParams(max_tokens=0),
+                       arrival_ns=time.monotonic_ns())
+        self._next_id += 1
+        self.sched.admit_open(seq)
+        self._open[seq.seq_id] = seq
+        return seq
+
+    @torch.inference_mode()
+    def feed_step(self, entries: list[tuple[Sequence, list[int], list[int]]]
+                  ) -> torch.Tensor | None:
+        """One engine step over given tokens: every (request, next tokens,
+        wanted offsets) entry runs in the same packed batch, from the cache
+        and state earlier steps left.  Returns fp32 logits [sum(wanted), V]
+        in entry order (None when nothing is wanted)."""
+        entries = [e for e in entries if e[1]]
+        if not entries:
+            return None
+        seqs = [e[0] for e in entries]
+        for seq, toks, _w in entries:
+            if seq.num_tokens + len(toks) > self.cfg.max_position:
+                raise ValueError("request exceeds model max_position")
+            self.sched.reserve(seq, len(toks))
+        ids_t, pos_t, md, cu_list = self._chunk_batch(
+            seqs, [s.num_tokens for s in seqs], [e[1] for e in entries])
+        rows = [cu_list[i] + w for i, e in enumerate(entries) for w in e[2]]
+        self.metrics["steps"] += 1
+        self.metrics["prefill_tokens"] += cu_list[-1]
+        for seq, toks, _w in entries:
+            seq.prompt_ids.extend(toks)
+            seq.num_prefilled = seq.num_tokens
+        rows_t = torch.tensor(rows or [0], dtype=torch.int32,
+                              device=self.device)
+        logits = self.model(ids_t, pos_t, self.kv, md, logit_rows=rows_t)
+        return logits.float() if rows else None
+
+    def close_request(self, seq: Sequence) -> None:
+        """Give back the pages and the state slot of an open request."""
+        if self._open.pop(seq.seq_id, None) is None:
+            return
+        self.sched.close_open(seq)
+        if self.state_slots is not None:
+            self.state_slots.release(seq)
+
     def _step_prefill_chunk(self) -> tuple[list[Sequence], list[int]]:
         """Prefill up to max_prefill_tokens across the pending prompts;
         sample only for prompts whose last chunk completed.
@@ -338,30 +478,11 @@ class LLMEngine:
             chunks.append(take)
             known.append(all_ids)
             budget -= take
-        ids, pos, slots, q_start = [], [], [], []
-        bt_rows = []
-        for seq, take, all_ids in zip(seqs, chunks, known):
-            np0 = seq.num_prefilled
-            ids.extend(all_ids[np0:np0 + take])
-            pos.extend(range(np0, np0 + take))
-            slots.extend(self._slot(seq, i) for i in range(np0, np0 + take))
-            q_start.append(np0)
-            row = torch.zeros(self.max_pages_per_seq, dtype=torch.int32)
-            row[:len(seq.pages)] = torch.tensor(seq.pages, dtype=torch.int32)
-            bt_rows.append(row)
-        self.metrics["prefill_tokens"] += len(ids)
-        cu_list = [0]
-        for ln in chunks:
-            cu_list.append(cu_list[-1] + ln)
-        cu = torch.tensor(cu_list, dtype=torch.int32, device=dev)
-        ids_t = torch.tensor(ids, dtype=torch.int32, device=dev)
-        pos_t = torch.tensor(pos, dtype=torch.int32, device=dev)
-        slots_t = torch.tensor(slots, dtype=torch.int64, device=dev)
-        md = AttnMetadata(is_prefill=True, slots=slots_t, cu_seqlens=cu,
-                          seq_lens=chunks,
-                          q_start=torch.tensor(q_start, dtype=torch.int32,
-                                               device=dev),
-                          block_table=torch.stack(bt_rows).to(dev))
+        ids_t, pos_t, md, cu_list = self._chunk_batch(
+            seqs, [s.num_prefilled for s in seqs],
+            [a[s.num_prefilled:s.num_prefilled + t]
+             for s, t, a in zip(seqs, chunks, known)])
+        self.metrics["prefill_tokens"] += cu_list[-1]
         done, done_rows = [], []
         for i, (seq, take, all_ids) in enumerate(zip(seqs, chunks, known)):
             seq.num_prefilled += take
@@ -375,7 +496,8 @@ class LLMEngine:
                        logit_rows=torch.zeros(1, dtype=torch.int32, device=dev))
             return [], []
         last_rows = torch.tensor(done_rows, dtype=torch.int32, device=dev)
-        logits = self.model(ids_t, pos_t, self.kv, md, logit_rows=last_rows)
+        logits = self._sampler_logits(
+            self.model(ids_t, pos_t, self.kv, md, logit_rows=last_rows))
         if any(s.sampling.json_mode for s in done):
             logits = logits + self._json_mask(done).to(logits.dtype)
         temps = torch.tensor([s.sampling.temperature for s in done],
@@ -391,6 +513,13 @@ class LLMEngine:
         if any(s.sampling.logprobs > 0 for s in done):
             self._attach_row_logprobs(done, logits, toks)
         return done, toks.cpu().tolist()
+
+    def _sampler_logits(self, logits: torch.Tensor) -> torch.Tensor:
+        """The sampling kernels read bf16 rows; models that hand back fp32
+        logits (soft-capped heads) are rounded once here."""
+        if self.is_gpu and logits.dtype != torch.bfloat16:
+            return logits.to(torch.bfloat16)
+        return logits
 
     def _attach_row_logprobs(self, seqs, logits, toks) -> None:
         """Per-row logprob reporting for eager paths (prefill-final and
@@ -752,7 +881,10 @@ class LLMEngine:
             h["temps"][i] = seq.sampling.temperature
             h["topk"][i] = seq.sampling.top_k
             h["topp"][i] = seq.sampling.top_p
+            if self.stateful:
+                h["sslot"][i] = self._state_slot(seq)
         for i in range(len(seqs), bs):  # dummy lanes -> null page 0
+            h["sslot"][i] = 0
             h["ids"][i] = 0
             h["pos"][i] = 0
             h["slots"][i] = 0
@@ -763,7 +895,8 @@ class LLMEngine:
             h["topp"][i] = 1.0
         d = self._dec
         nb = self.is_gpu
-        for k in ("ids", "pos", "slots", "lens", "temps", "topk", "topp"):
+        for k in ("ids", "pos", "slots", "lens", "temps", "topk", "topp",
+                  "sslot"):
             d[k][:bs].copy_(h[k][:bs], non_blocking=nb)
         d["bt"][:bs].copy_(h["bt"][:bs], non_blocking=nb)
 
@@ -773,7 +906,13 @@ class LLMEngine:
         md = AttnMetadata(is_prefill=False, slots=d["slots"][:bs],
                           block_table=d["bt"][:bs], seq_lens_t=d["lens"][:bs],
                           nsplit=nsplit, decode_scratch=scratch)
-        logits = self.model(d["ids"][:bs], d["pos"][:bs], self.kv, md)
+        if self.stateful:
+            md.state_slots = d["sslot"][:bs]
+            md.cu_seqlens = d["cu"][:bs + 1]
+            md.q_start = d["pos"][:bs]
+            md.row_seq = d["rowseq"][:bs]
+        logits = self._sampler_logits(
+            self.model(d["ids"][:bs], d["pos"][:bs], self.kv, md))
         if mask is not None:  # grammar-constrained rows (eager only)
             logits = logits + mask.to(logits.dtype)
         kw = {"topk": d["topk"][:bs], "topp": d["topp"][:bs]} if tkp else {}
@@ -789,7 +928,7 @@ class LLMEngine:
             d["lp_ids"][:bs] = ti.to(torch.int32)
 
     def _make_scratch(self, bs: int, nsplit: int):
-        if nsplit <= 1:
+        if nsplit <= 1 or not hasattr(self.cfg, "head_dim"):
             return None
         cfg = self.cfg
         G = cfg.num_heads // cfg.num_kv_heads

@@ -40,6 +40,47 @@ class PageAllocator:
         self.free_list.extend(pages)
 
 
+class SlotAllocator:
+    """Per-sequence state slots for models whose mixers carry state besides
+    paged K/V (recurrent matrices, token-shift rows).  Slot 0 is the null
+    slot of padded decode lanes, like page 0.  A slot is bound to one
+    admission of a sequence (seq_id, alloc_epoch): after a preemption the
+    sequence recomputes from position 0 and may land in any slot."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots           # usable slots (null excluded)
+        self.free_list = list(range(num_slots, 0, -1))
+        self.owner: dict[int, tuple[int, int]] = {}   # seq_id -> (epoch, slot)
+
+    @property
+    def num_free(self) -> int:
+        return len(self.free_list)
+
+    def slot_of(self, seq, live=None) -> int:
+        """The sequence's slot, taking a free one at (re)admission.  `live`
+        (seq_ids that may still run) lets stale owners be reclaimed."""
+        cur = self.owner.get(seq.seq_id)
+        if cur is not None and cur[0] == seq.alloc_epoch:
+            return cur[1]
+        if cur is not None:
+            self.free_list.append(cur[1])
+            del self.owner[seq.seq_id]
+        if not self.free_list and live is not None:
+            for sid in [s for s in self.owner if s not in live]:
+                self.free_list.append(self.owner.pop(sid)[1])
+        if not self.free_list:
+            raise MemoryError("state slots exhausted: more live sequences "
+                              "than max_num_seqs")
+        slot = self.free_list.pop()
+        self.owner[seq.seq_id] = (seq.alloc_epoch, slot)
+        return slot
+
+    def release(self, seq) -> None:
+        cur = self.owner.pop(seq.seq_id, None)
+        if cur is not None:
+            self.free_list.append(cur[1])
+
+
 @dataclass
 class SchedulerConfig:
     max_num_seqs: int = 64
@@ -180,6 +221,26 @@ class Scheduler:
     def note_token(self, seq: Sequence) -> None:
         """Interface parity with the native scheduler (token counting is
         implicit here via seq.num_tokens)."""
+
+    # -- caller-paced requests ---------------------------------------------
+    # A request whose tokens arrive from outside step by step (trace replay,
+    # teacher forcing): admitted with no tokens, pages reserved as tokens
+    # come, never queued, never preempted by schedule() (it is not in
+    # `running`).  Capacity errors surface to the caller.
+    def admit_open(self, seq: Sequence) -> None:
+        seq.pages = []
+        seq.alloc_epoch += 1
+        seq.status = SeqStatus.RUNNING
+
+    def reserve(self, seq: Sequence, ntokens: int) -> None:
+        """Pages for `ntokens` more tokens of an open request."""
+        need = self._pages_needed(seq.num_tokens + ntokens) - len(seq.pages)
+        if need > 0:
+            seq.pages.extend(self.alloc.alloc(need))
+
+    def close_open(self, seq: Sequence) -> None:
+        seq.status = SeqStatus.FINISHED
+        self.release(seq)
 
     def finish(self, seq: Sequence) -> None:
         seq.status = SeqStatus.FINISHED

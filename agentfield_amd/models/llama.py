@@ -132,6 +132,10 @@ class AttnMetadata:
              block_table [B,maxp] i32, slots [T] i64.
     Decode:  block_table [B,maxp] i32, seq_lens_t [B] i32, slots [B] i64,
              nsplit chosen by the engine.
+    Models that keep per-sequence state besides K/V (recurrent mixers, token
+    shift) also get state_slots [B] i32 and row_seq [T] i32 (the sequence
+    index of every row); for them a decode step is the packed-chunk layout
+    with one row per sequence (cu_seqlens = 0..B, q_start = position).
     """
     is_prefill: bool
     slots: torch.Tensor
@@ -142,6 +146,8 @@ class AttnMetadata:
     seq_lens_t: torch.Tensor | None = None
     nsplit: int = 1
     decode_scratch: tuple | None = None
+    state_slots: torch.Tensor | None = None
+    row_seq: torch.Tensor | None = None
 
 
 class KVCache:

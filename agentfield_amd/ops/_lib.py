@@ -82,6 +82,53 @@ def _declare(l: ctypes.CDLL) -> None:
         getattr(l, fn).restype = ctypes.c_int
 
 
+_MIX_PATH = Path(__file__).resolve().parent.parent / "libafmix.so"
+
+
+@functools.lru_cache(maxsize=1)
+def mixlib() -> ctypes.CDLL:
+    """The sequence-mixer kernel group (ops/seqmix.py).  Unlike the main
+    library it is compiled on first use when missing or older than its
+    sources — on a GPU box too — so a fresh checkout serving a hybrid model
+    builds exactly this group and nothing else."""
+    from agentfield_amd.build import build_mix
+    try:
+        build_mix(verbose=False)
+    except Exception as e:
+        if not _MIX_PATH.exists():
+            raise AfOpsError(f"libafmix.so could not be built: {e}") from e
+    cdll = ctypes.CDLL(str(_MIX_PATH))
+    _declare_mix(cdll)
+    return cdll
+
+
+def _declare_mix(l: ctypes.CDLL) -> None:
+    p, i, i64, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+    sig = {
+        "afm_embed": [p, p, p, p, i, i, i, p],
+        "afm_add_rows": [p, p, p, i, i, p],
+        "afm_dual_norm_shift": [p, p, p, p, p, p, p, p, p, p, p, p, p, f,
+                                i, i, i, p],
+        "afm_scatter_state": [p, p, p, p, i, i, p],
+        "afm_norm_rows": [p, p, p, p, f, i, i, i, i, p],
+        "afm_headnorm_gate": [p, p, p, p, f, i, i, i, i64, i, p],
+        "afm_polynorm": [p, p, p, f, i, i, i64, i, p],
+        "afm_gated_residual": [p, p, f, p, f, p, i64, p, p, p, i64, p,
+                               i, i, i, p],
+        "afm_softcap": [p, p, f, i64, i, p],
+        "afm_qk_norm_cache": [p, p, p, p, p, p, p, p, p, f, i, i, i, i, i, i,
+                              i, i, i64, i64, i64, i, p],
+        "afm_masked_attention": [p, p, p, p, p, p, p, f, i, i, i, i, i, i, i,
+                                 i, i, i64, i, p],
+        "afm_linear_scan": [p, p, p, p, p, p, p, p, p, p, p, p, p, f, f, f,
+                            i, i, i, i, i, i64, i64, i64, i64, i, p],
+    }
+    for name, args in sig.items():
+        fn = getattr(l, name)
+        fn.argtypes = args
+        fn.restype = ctypes.c_int
+
+
 def cur_stream() -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
