@@ -150,6 +150,23 @@ def engine(model: list[str] = ["llama-3-8b"], device: str = None,
     engine_main()
 
 
+@app.command("trace-run")
+def trace_run(model: str = typer.Option(..., help="checkpoint folder "
+                                        "(config.json + model.safetensors)"),
+              out: str = typer.Option(..., help="folder for <step>.f32"),
+              max_tokens: int = typer.Option(..., help="most tokens live "
+                                             "requests hold at any time"),
+              dtype: str = "bfloat16", device: str = None):
+    """Replay a token trace from stdin through the serving engine and write
+    the logits at the wanted places (no sampling).  Same as bin/trace_run."""
+    from .engine.replay import main as replay_main
+    argv = ["--model", model, "--out", out, "--max-tokens", str(max_tokens),
+            "--dtype", dtype]
+    if device:
+        argv += ["--device", device]
+    raise typer.Exit(replay_main(argv))
+
+
 AGENT_TEMPLATE = '''"""Agent scaffolded by `af init`."""
 from agentfield_amd.sdk import Agent
 

@@ -320,7 +320,8 @@ def get_runner(cfg: AIConfig) -> EngineRunner:
         # caching turns that repeated prefill into a block-table lookup
         # (opt out with AGENTFIELD_NO_PREFIX_CACHE=1)
         kw["prefix_cache"] = os.environ.get(
-            "AGENTFIELD_NO_PREFIX_CACHE") != "1"
+            "AGENTFIELD_NO_PREFIX_CACHE") != "1" and \
+            not getattr(model_cfg, "stateful", False)
         eng = LLMEngine(model_cfg, device=device, **kw)
         runner = EngineRunner(eng, tokenizer)
         _runners[key] = runner

@@ -11,6 +11,8 @@ import argparse
 import json
 import queue
 
+import os
+
 import torch
 from fastapi import FastAPI, Request
 from fastapi.responses import JSONResponse, StreamingResponse
@@ -562,8 +564,18 @@ def main():
             kw["eos_id"] = tokenizer.eos_id  # HF vocab EOS != byte EOS
         if args.max_prefill_tokens:
             kw["max_prefill_tokens"] = args.max_prefill_tokens
+        model = None
+        if name not in CONFIGS and os.path.isdir(name):
+            # a checkpoint directory: the registry picks the family by its
+            # config.json and loads the weights
+            from ..models import load_model
+            model = load_model(name, device=device,
+                               dtype=kw.get("dtype", torch.bfloat16))
+            cfg = model.cfg
+        else:
+            cfg = CONFIGS[name]
         eng = LLMEngine(
-            CONFIGS[name], device=device,
+            cfg, device=device, model=model,
             max_num_seqs=kw.pop("max_num_seqs", args.max_num_seqs),
             enable_graphs=not args.no_graphs and device.startswith("cuda"),
             spec_lookup=args.spec_lookup,

@@ -77,6 +77,14 @@ def parse_args():
                         "calls/s) because each step ends with a 128-response "
                         "stampede through the replica's event loop, so "
                         "in-process remains the default")
+    p.add_argument("--family-compare", action="store_true",
+                   help="instead of the default workload: engine-level "
+                        "prefill and decode token throughput of the hybrid "
+                        "(Reperax) family beside the Llama family at equal "
+                        "width / ff / depth, random weights; one JSON line "
+                        "per model and phase (single GPU)")
+    p.add_argument("--compare-pairs", default="reperax-1b:debug-1b",
+                   help="comma list of hybrid:llama config-name pairs")
     p.add_argument("--cp-workers", type=int, default=0,
                    help="control-plane worker processes (0 = auto)")
     return p.parse_args()
@@ -369,8 +377,93 @@ def run_step(eng: LLMEngine, rank: int, step: int, args) -> list[float]:
     return lat
 
 
+def _drive(eng: LLMEngine, prompts, gen_len: int):
+    """Run requests to completion; returns (prefill_s, prefill_tokens,
+    decode_s, decode_tokens) split by the kind of each engine step."""
+    sp = SamplingParams(max_tokens=gen_len, ignore_eos=True)
+    pending = set()
+    for p in prompts:
+        rid = eng.add_request(p, sp)
+        assert rid is not None
+        pending.add(rid)
+    m = eng.metrics
+    tp = td = 0.0
+    p0, d0 = m["prefill_tokens"], m["decode_tokens"]
+    sync = torch.cuda.synchronize if eng.is_gpu else (lambda: None)
+    while pending:
+        before = m["decode_steps"]
+        sync()
+        t0 = time.perf_counter()
+        eng.step()
+        sync()
+        dt = time.perf_counter() - t0
+        if m["decode_steps"] > before:
+            td += dt
+        else:
+            tp += dt
+        for rid in list(pending):
+            if eng.get_finished(rid) is not None:
+                pending.discard(rid)
+    return tp, m["prefill_tokens"] - p0, td, m["decode_tokens"] - d0
+
+
+def run_family_compare(args, device: str) -> None:
+    """Prefill and decode throughput of each config pair, engine-level."""
+    dtype = torch.bfloat16 if device.startswith("cuda") else torch.float32
+    small = not device.startswith("cuda")
+    plen = 64 if small else args.prompt_len * 4          # prefill prompts
+    nprefill = 2 if small else 8
+    dbatch = 4 if small else min(64, args.max_num_seqs)  # decode batch
+    dctx = 32 if small else args.prompt_len
+    dgen = 4 if small else args.gen_len
+    for pair in args.compare_pairs.split(","):
+        for name in pair.split(":"):
+            cfg = CONFIGS[name]
+            eng = LLMEngine(cfg, device=device, dtype=dtype,
+                            max_num_seqs=max(dbatch, nprefill),
+                            max_prefill_tokens=plen * nprefill,
+                            num_pages=(max(plen * nprefill,
+                                           dbatch * (dctx + dgen + 64))
+                                       // 64 + 64),
+                            enable_graphs=not args.no_graphs and not small,
+                            seed=0)
+            g = torch.Generator().manual_seed(7)
+
+            def prompts(n, ln):
+                return [torch.randint(0, cfg.vocab_size, (ln,),
+                                      generator=g).tolist() for _ in range(n)]
+            res = {}
+            for rep in range(args.warmup + args.steps):
+                tp, ntp, _, _ = _drive(eng, prompts(nprefill, plen), 1)
+                _, _, td, ntd = _drive(eng, prompts(dbatch, dctx), dgen)
+                if rep >= args.warmup:
+                    for k, v in (("tp", tp), ("ntp", ntp), ("td", td),
+                                 ("ntd", ntd)):
+                        res[k] = res.get(k, 0) + v
+            for phase, t, n, shape in (
+                    ("prefill", res["tp"], res["ntp"],
+                     {"prompts": nprefill, "prompt_len": plen}),
+                    ("decode", res["td"], res["ntd"],
+                     {"batch": dbatch, "context": dctx, "gen_len": dgen})):
+                print(json.dumps({
+                    "metric": f"{phase}_tokens_per_sec",
+                    "value": round(n / t, 1), "unit": "tokens/s",
+                    "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                    "higher_is_better": True,
+                    "dtype": "bf16" if dtype == torch.bfloat16 else "fp32",
+                    "data": "synthetic",
+                    "config": {"model": name, **shape}}), flush=True)
+            del eng
+            if device.startswith("cuda"):
+                torch.cuda.empty_cache()
+
+
 def main():
     args = parse_args()
+    if args.family_compare:
+        run_family_compare(args, args.device or (
+            "cuda" if torch.cuda.is_available() else "cpu"))
+        return
     world = int(os.environ.get("WORLD_SIZE", "1"))
     rank = int(os.environ.get("RANK", "0"))
     local_rank = int(os.environ.get("LOCAL_RANK", "0"))
