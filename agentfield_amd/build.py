@@ -41,7 +41,7 @@ HIP_SOURCES = [
 # Kernel groups that build into their own small library, so a process that
 # serves only one model family compiles (and loads) only what it runs.
 # libafmix.so: sequence-mixer op set (ops/seqmix.py).
-MIX_SOURCES = ["mix_glue.hip", "mix_seq.hip"]
+MIX_SOURCES = ["mix_glue.hip", "mix_seq.hip", "mix_attn_mfma.hip"]
 MIX_LIB = PKG_DIR / "libafmix.so"
 
 # hipcc -O3 may otherwise fuse scalar float code into packed-fp32 VALU ops
@@ -68,6 +68,18 @@ def build_afops(force: bool = False, verbose: bool = True) -> Path:
     return _build_lib(LIB, HIP_SOURCES, force, verbose)
 
 
+def _run(cmd, verbose: bool) -> None:
+    if verbose:
+        print("[afops]", " ".join(cmd), file=sys.stderr)
+        subprocess.run(cmd, check=True)
+        return
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                       text=True)
+    if r.returncode != 0:
+        sys.stderr.write(r.stdout)
+        raise subprocess.CalledProcessError(r.returncode, cmd)
+
+
 def _build_lib(lib: Path, sources, force: bool, verbose: bool) -> Path:
     if not force and not _needs_build(lib, sources):
         return lib
@@ -87,19 +99,15 @@ def _build_lib(lib: Path, sources, force: bool, verbose: bool) -> Path:
             HIPCC, f"--offload-arch={ARCH}", *HIP_FLAGS,
             "-c", str(sp), "-o", str(op),
         ]
-        if verbose:
-            print("[afops]", " ".join(cmd), file=sys.stderr)
-        subprocess.run(cmd, check=True)
+        _run(cmd, verbose)
     # link to a temporary name and rename: a concurrent process never maps a
     # half-written library
     fd, tmp = tempfile.mkstemp(dir=str(lib.parent), prefix=lib.name + ".")
     os.close(fd)
     cmd = [HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC",
            *[str(o) for o in objs], "-o", tmp]
-    if verbose:
-        print("[afops]", " ".join(cmd), file=sys.stderr)
     try:
-        subprocess.run(cmd, check=True)
+        _run(cmd, verbose)
         os.chmod(tmp, 0o755)
         os.replace(tmp, lib)
     finally:

@@ -1,0 +1,246 @@
+// Masked (causal / chunk-local / banded) paged prefill attention on the
+// matrix cores, bf16 storage, for head sizes up to 128 that need not be a
+// power of two.  Scores, mask, softmax statistics and the output accumulator
+// are fp32; Q.K^T and P.V run as MFMA 16x16x32 bf16.
+//
+// Workgroup = 64 consecutive chunk rows of one sequence x one query head;
+// wave w owns rows 16w..16w+15.  Key/value tiles of 64 positions are staged
+// once per workgroup through LDS: K row-major (rows padded by 16 B), V
+// transposed [d][token] with token pairs packed into 32-bit writes, the
+// wave's probabilities round-trip through a private LDS tile to turn the
+// MFMA C layout into an A fragment.  Head sizes are zero-padded to the
+// template extent (DKC*32 for q/k, DVT*16 for v).  Only key tiles that
+// intersect the rows' visible range are visited: for chunk-local attention
+// that is at most chunk/64 + 1 tiles per workgroup.
+//
+// Fragment layouts of v_mfma_f32_16x16x32_bf16 (64-lane wave):
+//   A: lane holds A[m = lane&15][k = (lane>>4)*8 + j], j = 0..7
+//   B: lane holds B[k = (lane>>4)*8 + j][n = lane&15]
+//   C: lane reg r holds C[m = (lane>>4)*4 + r][n = lane&15]
+#include "common.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+
+__device__ __forceinline__ bf16x8 as_bf16x8(s16x8 v) {
+  union { s16x8 s; bf16x8 b; } u;
+  u.s = v;
+  return u.b;
+}
+
+// 8 consecutive bf16 starting at element e0 of a row of n valid elements;
+// elements >= n read as zero.  VEC: rows and e0 are 16-byte aligned and n is
+// a multiple of 8, so a group is either fully inside or fully outside.
+template <bool VEC>
+__device__ __forceinline__ s16x8 load8(const u16* row, int e0, int n) {
+  s16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (VEC) {
+    if (e0 < n) v = *reinterpret_cast<const s16x8*>(row + e0);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (e0 + j < n) v[j] = (short)row[e0 + j];
+  }
+  return v;
+}
+
+template <int DKC, int DVT, bool VEC>
+__global__ void __launch_bounds__(256) attn_prefill_mfma_kernel(
+    u16* __restrict__ out, const u16* __restrict__ q,
+    const u16* __restrict__ kc, const u16* __restrict__ vc,
+    const i32* __restrict__ bt, const i32* __restrict__ cu,
+    const i32* __restrict__ q_start, const i32* __restrict__ tile_seq,
+    const i32* __restrict__ tile_q0, float scale, int H, int G, int dk, int dv,
+    int page, int maxp, int chunk, int window, i64 ldq) {
+  constexpr int KS = DKC * 32 + 8;   // K row stride in LDS (elements)
+  constexpr int VS = 72;             // V^T / P row stride (64 tokens + pad)
+  __shared__ u16 k_lds[64 * KS];
+  __shared__ u16 v_lds[DVT * 16 * VS];
+  __shared__ u16 p_lds[4 * 16 * VS];
+
+  const int tile = blockIdx.x, h = blockIdx.y;
+  const int g = h / (H / G);
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int b = tile_seq[tile];
+  const int r0 = cu[b];
+  const int len = cu[b + 1] - r0;
+  const int q0 = tile_q0[tile];                // first chunk row of the tile
+  const int nrows = min(64, len - q0);
+  const int p0 = q_start[b] + q0;              // position of the first row
+  const int p_last = p0 + nrows - 1;
+  const i32* btr = bt + (size_t)b * maxp;
+
+  // visible key range of the whole tile: row p0 reaches back the farthest
+  int lo = 0;
+  if (chunk > 0) lo = (p0 / chunk) * chunk;
+  if (window > 0) lo = max(lo, p0 - window + 1);
+
+  // this wave's rows
+  const int wrow0 = wid * 16;
+  const bool wave_live = wrow0 < nrows;
+  const int wp0 = p0 + wrow0;                              // first position
+  const int wp_last = min(p0 + wrow0 + 15, p_last);        // last position
+
+  s16x8 q_frag[DKC];
+  {
+    const int row = min(q0 + wrow0 + (lane & 15), len - 1);
+    const u16* qr = q + (size_t)(r0 + row) * ldq + (size_t)h * dk;
+#pragma unroll
+    for (int c = 0; c < DKC; ++c)
+      q_frag[c] = load8<VEC>(qr, c * 32 + (lane >> 4) * 8, dk);
+  }
+  float m[4], l[4];
+  f32x4 o_acc[DVT];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) { m[r] = AF_NEG_INF; l[r] = 0.f; }
+#pragma unroll
+  for (int dt = 0; dt < DVT; ++dt) o_acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  u16* pw = p_lds + wid * 16 * VS;
+
+  for (int kv0 = lo; kv0 <= p_last; kv0 += 64) {
+    __syncthreads();   // fragment reads of the previous tile are done
+    // ---- stage K: 64 tokens x DKC*4 groups of 8 ----
+    for (int i = threadIdx.x; i < 64 * DKC * 4; i += 256) {
+      const int tok = i / (DKC * 4), e0 = (i % (DKC * 4)) * 8;
+      const int j = kv0 + tok;
+      s16x8 v8 = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (j <= p_last) {
+        const u16* kr = kc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * dk;
+        v8 = load8<VEC>(kr, e0, dk);
+      }
+      *reinterpret_cast<s16x8*>(k_lds + tok * KS + e0) = v8;
+    }
+    // ---- stage V transposed: token pairs -> one 32-bit write per d ----
+    for (int i = threadIdx.x; i < 32 * DVT * 2; i += 256) {
+      const int tp = i % 32, e0 = (i / 32) * 8;
+      const int j0 = kv0 + tp * 2;
+      s16x8 a = {0, 0, 0, 0, 0, 0, 0, 0}, c8 = a;
+      if (j0 <= p_last)
+        a = load8<VEC>(vc + (((size_t)btr[j0 / page] * G + g) * page + (j0 % page)) * dv, e0, dv);
+      if (j0 + 1 <= p_last)
+        c8 = load8<VEC>(vc + (((size_t)btr[(j0 + 1) / page] * G + g) * page + ((j0 + 1) % page)) * dv, e0, dv);
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) {
+        const uint32_t packed = (uint32_t)(unsigned short)a[jj] |
+                                ((uint32_t)(unsigned short)c8[jj] << 16);
+        *reinterpret_cast<uint32_t*>(v_lds + (e0 + jj) * VS + tp * 2) = packed;
+      }
+    }
+    __syncthreads();
+    // keys of this tile that any row of the wave may see
+    if (!wave_live || kv0 > wp_last) continue;
+    if (window > 0 && kv0 + 63 <= wp0 - window) continue;
+
+    // ---- S = Q K^T: four 16-key sub-tiles ----
+    f32x4 s_acc[4];
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+      s_acc[st] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const u16* krow = k_lds + (st * 16 + (lane & 15)) * KS + (lane >> 4) * 8;
+#pragma unroll
+      for (int c = 0; c < DKC; ++c) {
+        const s16x8 kf = *reinterpret_cast<const s16x8*>(krow + c * 32);
+        s_acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            as_bf16x8(q_frag[c]), as_bf16x8(kf), s_acc[st], 0, 0, 0);
+      }
+    }
+    // ---- mask + online softmax; reg r is row (lane>>4)*4 + r ----
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int p = wp0 + (lane >> 4) * 4 + r;
+      int rlo = 0;
+      if (chunk > 0) rlo = (p / chunk) * chunk;
+      if (window > 0) rlo = max(rlo, p - window + 1);
+      float sr[4];
+      float tmax = AF_NEG_INF;
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        const int j = kv0 + st * 16 + (lane & 15);
+        sr[st] = (j <= p && j >= rlo) ? s_acc[st][r] * scale : AF_NEG_INF;
+        tmax = fmaxf(tmax, sr[st]);
+      }
+      tmax = group16_max_f32(tmax);
+      const float mn = fmaxf(m[r], tmax);
+      const float corr = (m[r] <= AF_NEG_INF) ? 0.f : __expf(m[r] - mn);
+      float psum = 0.f;
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        sr[st] = (sr[st] <= AF_NEG_INF) ? 0.f : __expf(sr[st] - mn);
+        psum += sr[st];
+        s_acc[st][r] = sr[st];
+      }
+      l[r] = l[r] * corr + group16_sum_f32(psum);
+      m[r] = mn;
+#pragma unroll
+      for (int dt = 0; dt < DVT; ++dt) o_acc[dt][r] *= corr;
+    }
+    // ---- P: C layout -> A fragments through the wave's LDS tile ----
+#pragma unroll
+    for (int st = 0; st < 4; ++st)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        pw[((lane >> 4) * 4 + r) * VS + st * 16 + (lane & 15)] = f2bf(s_acc[st][r]);
+    __builtin_amdgcn_wave_barrier();
+    const s16x8 pf0 = *reinterpret_cast<const s16x8*>(pw + (lane & 15) * VS + (lane >> 4) * 8);
+    const s16x8 pf1 = *reinterpret_cast<const s16x8*>(pw + (lane & 15) * VS + 32 + (lane >> 4) * 8);
+    __builtin_amdgcn_wave_barrier();
+    // ---- O += P V ----
+#pragma unroll
+    for (int dt = 0; dt < DVT; ++dt) {
+      const u16* vrow = v_lds + (dt * 16 + (lane & 15)) * VS + (lane >> 4) * 8;
+      const s16x8 vf0 = *reinterpret_cast<const s16x8*>(vrow);
+      const s16x8 vf1 = *reinterpret_cast<const s16x8*>(vrow + 32);
+      o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+          as_bf16x8(pf0), as_bf16x8(vf0), o_acc[dt], 0, 0, 0);
+      o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+          as_bf16x8(pf1), as_bf16x8(vf1), o_acc[dt], 0, 0, 0);
+    }
+  }
+
+  if (!wave_live) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = q0 + wrow0 + (lane >> 4) * 4 + r;
+    if (row >= len) continue;
+    const float inv = l[r] > 0.f ? 1.0f / l[r] : 0.f;
+    u16* op = out + ((size_t)(r0 + row) * H + h) * dv;
+#pragma unroll
+    for (int dt = 0; dt < DVT; ++dt) {
+      const int d = dt * 16 + (lane & 15);
+      if (d < dv) op[d] = f2bf(o_acc[dt][r] * inv);
+    }
+  }
+}
+
+}  // namespace
+
+// q [T, H*dk] bf16 rows at stride ldq; caches [P, G, page, dk|dv] bf16;
+// tile map (tile_seq, tile_q0): workgroup i covers chunk rows
+// [q0, q0 + 64) of sequence tile_seq[i].  out [T, H*dv] bf16.
+AF_EXPORT int afm_attn_prefill_mfma(
+    void* out, const void* q, const void* kc, const void* vc, const void* bt,
+    const void* cu, const void* q_start, const void* tile_seq,
+    const void* tile_q0, float scale, int ntiles, int H, int G, int dk, int dv,
+    int page, int maxp, int chunk, int window, i64 ldq, void* stream) {
+  if (ntiles == 0) return 0;
+  if (G <= 0 || H % G || dk < 1 || dv < 1 || dk > 128 || dv > 128) return 9003;
+  const bool vec = (dk % 8 == 0) && (dv % 8 == 0) && (ldq % 8 == 0) &&
+                   ((uintptr_t)q % 16 == 0) && ((uintptr_t)kc % 16 == 0) &&
+                   ((uintptr_t)vc % 16 == 0);
+  dim3 grid(ntiles, H), blk(256);
+  hipStream_t s = (hipStream_t)stream;
+#define APM(DKC, DVT, VEC)                                                     \
+  attn_prefill_mfma_kernel<DKC, DVT, VEC><<<grid, blk, 0, s>>>(                \
+      (u16*)out, (const u16*)q, (const u16*)kc, (const u16*)vc,                \
+      (const i32*)bt, (const i32*)cu, (const i32*)q_start,                     \
+      (const i32*)tile_seq, (const i32*)tile_q0, scale, H, G, dk, dv, page,    \
+      maxp, chunk, window, ldq)
+  const bool small = dk <= 64 && dv <= 64;
+  if (small && vec) APM(2, 4, true);
+  else if (small) APM(2, 4, false);
+  else if (vec) APM(4, 8, true);
+  else APM(4, 8, false);
+#undef APM
+  return af_last_err();
+}

@@ -136,11 +136,15 @@ __global__ void __launch_bounds__(256) masked_attention_kernel(
 
 // ------------------------------------------------------------- linear scan
 // Workgroup = (sequence, head, 32-column tile of dv); 256 threads = 8 row
-// groups x 32 columns.  Thread (r, c) keeps rows r, r+8, ... of column c of
-// the state in registers (RP rows).  Tokens are walked serially; q/k/decay
-// rows are staged through double-buffered LDS (rotary + scaling applied on
-// the way in), partial outputs are reduced across the 8 row groups through a
-// double-buffered LDS tile one token late, so a token costs one barrier.
+// groups x 32 columns.  Thread (r, c) keeps RP consecutive rows
+// r*RP .. r*RP+RP-1 of column c of the state in registers.  Tokens are
+// walked serially in blocks of TB: the block's q / k / decay rows are staged
+// into LDS at once (rotary + scaling applied on the way in), every thread
+// then advances its rows through the TB tokens without synchronising and
+// leaves one partial output per token in LDS, and the 8 partials of each
+// (token, column) are summed after one more barrier: two barriers per TB
+// tokens, the recurrence itself strictly token by token in fp32 — so results
+// are bit-identical however a sequence is cut into chunks.
 template <typename S, int RP>
 __global__ void __launch_bounds__(256) linear_scan_kernel(
     float* __restrict__ out, float* __restrict__ state,
@@ -151,88 +155,105 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
     const i32* __restrict__ q_start, const i32* __restrict__ sslot,
     float q_scale, float k_scale, float inv_tau, int H, int dk, int dv,
     int rot, i64 ldq, i64 ldk, i64 ldv, i64 ldz) {
-  extern __shared__ float smem[];  // [2][3*dk] + [2][8*32]
+  constexpr int DKP = 8 * RP;          // padded rows: zeros beyond dk
+  constexpr int SCAN_TB = RP >= 32 ? 8 : 16;  // keeps LDS under 64 KB
+  extern __shared__ float smem[];      // [TB][3][DKP] + [TB][8][32] + [TB][32]
   const int b = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 32;
   const int t0 = cu[b], t1 = cu[b + 1];
   if (t1 <= t0) return;
   const int r = threadIdx.x >> 5, cc = threadIdx.x & 31;
   const int c = c0 + cc;
   const bool cok = c < dv;
-  float* stage = smem;                 // [2][3][dk]: q, k, decay
-  float* red = smem + 6 * dk;          // [2][8][32]
+  float* stage = smem;                         // [TB][3][DKP]: q, k, decay
+  float* part = smem + SCAN_TB * 3 * DKP;      // [TB][8][32]
+  float* vs = part + SCAN_TB * 256;            // [TB][32]
   float* sbase = state + (((size_t)sslot[b] * H + h) * dk) * dv;
   float st[RP];
   const bool fresh = q_start[b] == 0;
 #pragma unroll
   for (int ii = 0; ii < RP; ++ii) {
-    const int i = r + 8 * ii;
+    const int i = r * RP + ii;
     st[ii] = (!fresh && cok && i < dk) ? sbase[(size_t)i * dv + c] : 0.f;
   }
   const float hd = head_decay ? head_decay[h] : 1.0f;
   const int half = rot >> 1;
-  for (int t = t0; t < t1; ++t) {
-    float* sq = stage + (size_t)((t - t0) & 1) * 3 * dk;
-    float* sk = sq + dk;
-    float* sa = sk + dk;
-    const S* qr = q + (size_t)t * ldq + (size_t)h * dk;
-    const S* kr = k + (size_t)t * ldk + (size_t)h * dk;
-    const float posf = (float)positions[t];
-    for (int i = threadIdx.x; i < dk; i += 256) {
-      float qv = ldf<S>(qr + i), kv = ldf<S>(kr + i);
-      if (i < rot) {
-        const bool lowh = i < half;
-        const int fi = lowh ? i : i - half;
-        const int pi = lowh ? i + half : i - half;
-        const float ang = posf * inv_freq[fi];
-        const float cs = cosf(ang), sn = sinf(ang);
-        const float qp = ldf<S>(qr + pi), kp = ldf<S>(kr + pi);
-        // pair (u, w) -> (u cos - w sin, w cos + u sin)
-        qv = lowh ? qv * cs - qp * sn : qv * cs + qp * sn;
-        kv = lowh ? kv * cs - kp * sn : kv * cs + kp * sn;
-      }
-      sq[i] = qv * q_scale;
-      sk[i] = kv * k_scale;
-      float a = hd;
-      if (zl) {
-        const float z = ldf<S>(zl + (size_t)t * ldz + (size_t)h * dk + i) + zbias[(size_t)h * dk + i];
-        // log(sigmoid(z)) = -softplus(-z), evaluated without overflow
-        const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
-        a = expf(ls * inv_tau);
-      }
-      sa[i] = a;
-    }
-    const float vv = cok ? ldf<S>(v + (size_t)t * ldv + (size_t)h * dv + c) : 0.f;
-    __syncthreads();
-    if (t > t0 && r == 0 && cok) {
-      const float* rd = red + (size_t)((t - 1 - t0) & 1) * 256;
-      float o = 0.f;
-#pragma unroll
-      for (int rr = 0; rr < 8; ++rr) o += rd[rr * 32 + cc];
-      out[(size_t)(t - 1) * H * dv + (size_t)h * dv + c] = o;
-    }
-    float part = 0.f;
-#pragma unroll
-    for (int ii = 0; ii < RP; ++ii) {
-      const int i = r + 8 * ii;
+  for (int tb = t0; tb < t1; tb += SCAN_TB) {
+    const int nt = min(SCAN_TB, t1 - tb);
+    // ---- stage nt tokens: q, k (rotated, scaled) and decay rows ----
+    for (int e = threadIdx.x; e < nt * DKP; e += 256) {
+      const int tt = e / DKP, i = e % DKP;
+      float* row = stage + (size_t)tt * 3 * DKP;
+      float qv = 0.f, kv = 0.f, a = 0.f;
       if (i < dk) {
-        st[ii] = sa[i] * st[ii] + sk[i] * vv;
-        part += st[ii] * sq[i];
+        const int t = tb + tt;
+        const S* qr = q + (size_t)t * ldq + (size_t)h * dk;
+        const S* kr = k + (size_t)t * ldk + (size_t)h * dk;
+        qv = ldf<S>(qr + i);
+        kv = ldf<S>(kr + i);
+        if (i < rot) {
+          const bool lowh = i < half;
+          const int fi = lowh ? i : i - half;
+          const int pi = lowh ? i + half : i - half;
+          const float ang = (float)positions[t] * inv_freq[fi];
+          const float cs = cosf(ang), sn = sinf(ang);
+          const float qp = ldf<S>(qr + pi), kp = ldf<S>(kr + pi);
+          // pair (u, w) -> (u cos - w sin, w cos + u sin)
+          qv = lowh ? qv * cs - qp * sn : qv * cs + qp * sn;
+          kv = lowh ? kv * cs - kp * sn : kv * cs + kp * sn;
+        }
+        qv *= q_scale;
+        kv *= k_scale;
+        a = hd;
+        if (zl) {
+          const float z = ldf<S>(zl + (size_t)t * ldz + (size_t)h * dk + i) +
+                          zbias[(size_t)h * dk + i];
+          // log(sigmoid(z)) = -softplus(-z), evaluated without overflow
+          const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
+          a = expf(ls * inv_tau);
+        }
+      }
+      row[i] = qv;
+      row[DKP + i] = kv;
+      row[2 * DKP + i] = a;
+    }
+    for (int e = threadIdx.x; e < nt * 32; e += 256) {
+      const int tt = e >> 5, ci = c0 + (e & 31);
+      vs[e] = ci < dv ? ldf<S>(v + (size_t)(tb + tt) * ldv + (size_t)h * dv + ci) : 0.f;
+    }
+    __syncthreads();
+    // ---- advance this thread's rows through the block, token by token ----
+    for (int tt = 0; tt < nt; ++tt) {
+      const float* sq = stage + (size_t)tt * 3 * DKP + r * RP;
+      const float* sk = sq + DKP;
+      const float* sa = sk + DKP;
+      const float vv = vs[tt * 32 + cc];
+      float p = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < RP; ++ii) {
+        st[ii] = sa[ii] * st[ii] + sk[ii] * vv;
+        p += st[ii] * sq[ii];
+      }
+      part[tt * 256 + r * 32 + cc] = p;
+    }
+    __syncthreads();
+    // ---- o[t][c] = sum of the 8 row-group partials ----
+    for (int e = threadIdx.x; e < nt * 32; e += 256) {
+      const int tt = e >> 5, ci = e & 31;
+      if (c0 + ci < dv) {
+        const float* pr = part + tt * 256 + ci;
+        float o = 0.f;
+#pragma unroll
+        for (int rr = 0; rr < 8; ++rr) o += pr[rr * 32];
+        out[(size_t)(tb + tt) * H * dv + (size_t)h * dv + c0 + ci] = o;
       }
     }
-    red[(size_t)((t - t0) & 1) * 256 + r * 32 + cc] = part;
-  }
-  __syncthreads();
-  if (r == 0 && cok) {
-    const float* rd = red + (size_t)((t1 - 1 - t0) & 1) * 256;
-    float o = 0.f;
-#pragma unroll
-    for (int rr = 0; rr < 8; ++rr) o += rd[rr * 32 + cc];
-    out[(size_t)(t1 - 1) * H * dv + (size_t)h * dv + c] = o;
+    // the next block's staging writes `stage`/`vs`, last read before the
+    // barrier above; its partials are written after the next barrier
   }
   if (cok) {
 #pragma unroll
     for (int ii = 0; ii < RP; ++ii) {
-      const int i = r + 8 * ii;
+      const int i = r * RP + ii;
       if (i < dk) sbase[(size_t)i * dv + c] = st[ii];
     }
   }
@@ -312,8 +333,9 @@ static int launch_scan(float* out, float* state, const void* q, const void* k,
                        float inv_tau, int B, int H, int dk, int dv, int rot,
                        i64 ldq, i64 ldk, i64 ldv, i64 ldz, hipStream_t s) {
   dim3 grid(B, H, (dv + 31) / 32);
-  const size_t sm = (size_t)(6 * dk + 512) * sizeof(float);
   const int rp = (dk + 7) / 8;
+  const int rpp = rp <= 4 ? 4 : rp <= 8 ? 8 : rp <= 16 ? 16 : 32;
+  const size_t sm = (size_t)(rpp >= 32 ? 8 : 16) * (3 * 8 * rpp + 256 + 32) * sizeof(float);
 #define SCAN(RP)                                                             \
   linear_scan_kernel<S, RP><<<grid, 256, sm, s>>>(                           \
       out, state, (const S*)q, (const S*)k, (const S*)v, (const S*)zl, zbias, \

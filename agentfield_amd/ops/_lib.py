@@ -120,6 +120,8 @@ def _declare_mix(l: ctypes.CDLL) -> None:
                               i, i, i64, i64, i64, i, p],
         "afm_masked_attention": [p, p, p, p, p, p, p, f, i, i, i, i, i, i, i,
                                  i, i, i64, i, p],
+        "afm_attn_prefill_mfma": [p, p, p, p, p, p, p, p, p, f, i, i, i, i, i,
+                                  i, i, i, i, i64, p],
         "afm_linear_scan": [p, p, p, p, p, p, p, p, p, p, p, p, p, f, f, f,
                             i, i, i, i, i, i64, i64, i64, i64, i, p],
     }

@@ -26,6 +26,9 @@ import torch
 from . import _lib
 
 _DT = {torch.bfloat16: 0, torch.float32: 1}
+# a step whose longest row chunk reaches this many rows runs bf16 attention
+# through the MFMA tile kernel; shorter steps (decode) use one wave per row
+MFMA_MIN_ROWS = 16
 
 
 def _gpu(t: torch.Tensor) -> bool:
@@ -228,6 +231,26 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
             out[t] = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), vv)
         return out.view(T, H * dv).to(q.dtype)
     out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+    lens = getattr(md, "seq_lens", None)
+    if (q.dtype == torch.bfloat16 and lens is not None and dk <= 128
+            and dv <= 128 and max(lens) >= MFMA_MIN_ROWS):
+        # prompt portions: 64-row tiles on the matrix cores
+        ts, tq = [], []
+        for b, ln in enumerate(lens):
+            for q0 in range(0, ln, 64):
+                ts.append(b)
+                tq.append(q0)
+        tile_seq = torch.tensor(ts, dtype=torch.int32, device=q.device)
+        tile_q0 = torch.tensor(tq, dtype=torch.int32, device=q.device)
+        rc = _L().afm_attn_prefill_mfma(
+            _lib.ptr(out), _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vcache),
+            _lib.ptr(md.block_table), _lib.ptr(md.cu_seqlens),
+            _lib.ptr(md.q_start), _lib.ptr(tile_seq), _lib.ptr(tile_q0),
+            float(scale), len(ts), H, G, dk, dv, page,
+            md.block_table.shape[1], int(chunk), int(window), _rowstride(q),
+            _lib.cur_stream())
+        _lib.check(rc, "afm_attn_prefill_mfma")
+        return out
     rc = _L().afm_masked_attention(
         _lib.ptr(out), _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vcache),
         _lib.ptr(md.block_table), _lib.ptr(md.row_seq), _lib.ptr(positions),

@@ -156,7 +156,8 @@ def md_for(chunks, starts, slots, device, page=8, pages_per_seq=16):
                          state_slots=t(slots, torch.int32),
                          row_seq=t(rowseq, torch.int32),
                          block_table=bt.to(device),
-                         slots=t(kvslots, torch.int64))
+                         slots=t(kvslots, torch.int64),
+                         seq_lens=list(chunks), is_prefill=True)
     return md, t(pos, torch.int32)
 
 
@@ -204,7 +205,7 @@ def test_dual_norm_shift_and_state(device, dtype):
 def test_chunk_attention_alone(device, dtype, shape):
     H, G, dk, dv, chunk = shape
     torch.manual_seed(2)
-    W, T, page = 24, 29, 8
+    W, T, page = 24, 133, 8
     h = torch.randn(T, W).to(dtype)
     Wq, Wk, Wv = (torch.randn(n, W).to(dtype) / 5
                   for n in (H * dk, G * dk, G * dv))
@@ -218,8 +219,10 @@ def test_chunk_attention_alone(device, dtype, shape):
     vc = torch.zeros(20, G, page, dv, dtype=dtype, device=device)
     hd = h.to(device)
     got = []
-    for lo, hi in ((0, 11), (11, 13), (13, 14), (14, 29)):
-        md, pos = md_for([hi - lo], [lo], [1], device, page)
+    # short portions run one wave per row, long ones the 64-row tile kernel
+    for lo, hi in ((0, 11), (11, 13), (13, 14), (14, 31), (31, 112),
+                   (112, 133)):
+        md, pos = md_for([hi - lo], [lo], [1], device, page, 18)
         q = sm.qk_norm_cache(hd[lo:hi] @ Wq.to(device).T,
                              hd[lo:hi] @ Wk.to(device).T,
                              hd[lo:hi] @ Wv.to(device).T, gq.to(device),
@@ -230,7 +233,8 @@ def test_chunk_attention_alone(device, dtype, shape):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-def test_chunk_edge_one_key_stands_out(device):
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_chunk_edge_one_key_stands_out(device, dtype):
     """A query that matches one key overwhelmingly returns that key's value
     when the key is the first of the query's chunk, and none of it when the
     key is the last of the chunk before."""
@@ -246,15 +250,16 @@ def test_chunk_edge_one_key_stands_out(device):
         kk, vv = k.clone(), v.clone()
         kk[key_pos] = u
         vv[key_pos] = 5.0
-        kc = torch.zeros(8, 1, page, dk, device=device)
-        vc = torch.zeros(8, 1, page, dv, device=device)
+        kc = torch.zeros(8, 1, page, dk, device=device, dtype=dtype)
+        vc = torch.zeros(8, 1, page, dv, device=device, dtype=dtype)
         md, pos = md_for([T], [0], [1], device, page)
         q = torch.randn(T, dk) * 0.1
         q[query_pos] = u
-        qn = sm.qk_norm_cache(q.to(device), kk.to(device), vv.to(device),
-                              None, None, 1e-5, kc, vc, md.slots)
+        qn = sm.qk_norm_cache(q.to(device, dtype), kk.to(device, dtype),
+                              vv.to(device, dtype), None, None, 1e-5, kc, vc,
+                              md.slots)
         o = sm.masked_attention(qn, kc, vc, md, pos, 1.0, 1, chunk=chunk)
-        row = o[query_pos].cpu()
+        row = o[query_pos].cpu().float()
         if seen:
             assert torch.allclose(row, torch.full((dv,), 5.0), atol=1e-3)
         else:
@@ -263,7 +268,8 @@ def test_chunk_edge_one_key_stands_out(device):
         md1, pos1 = md_for([1], [query_pos], [1], device, page)
         o1 = sm.masked_attention(qn[query_pos:query_pos + 1], kc, vc, md1,
                                  pos1, 1.0, 1, chunk=chunk)
-        assert torch.allclose(o1[0].cpu(), row, atol=1e-5)
+        assert torch.allclose(o1[0].cpu().float(), row,
+                              atol=1e-5 if dtype == torch.float32 else 3e-2)
 
 
 @pytest.mark.parametrize("device", DEVICES)
