@@ -17,6 +17,41 @@ template <typename S> __device__ __forceinline__ void stf(S* p, float v);
 template <> __device__ __forceinline__ void stf<u16>(u16* p, float v) { *p = f2bf(v); }
 template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
 
+// 4 consecutive elements (8 B of bf16 / 16 B of fp32); callers guarantee the
+// alignment (row lengths and strides multiples of 4, 16-byte aligned bases).
+template <typename S> __device__ __forceinline__ void ld4(const S* p, float (&o)[4]);
+template <> __device__ __forceinline__ void ld4<u16>(const u16* p, float (&o)[4]) {
+  const s16x4 v = *reinterpret_cast<const s16x4*>(p);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = bf2f((u16)v[j]);
+}
+template <> __device__ __forceinline__ void ld4<float>(const float* p, float (&o)[4]) {
+  const f32x4 v = *reinterpret_cast<const f32x4*>(p);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = v[j];
+}
+template <typename S> __device__ __forceinline__ void st4(S* p, const float (&o)[4]);
+template <> __device__ __forceinline__ void st4<u16>(u16* p, const float (&o)[4]) {
+  s16x4 v;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = (short)f2bf(o[j]);
+  *reinterpret_cast<s16x4*>(p) = v;
+}
+template <> __device__ __forceinline__ void st4<float>(float* p, const float (&o)[4]) {
+  *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+}
+// V = 4: vector accesses; V = 1: scalar fallback for odd sizes.
+template <typename S, int V>
+__device__ __forceinline__ void ldv(const S* p, float (&o)[4]) {
+  if (V == 4) ld4<S>(p, o);
+  else { o[0] = ldf<S>(p); o[1] = o[2] = o[3] = 0.f; }
+}
+template <typename S, int V>
+__device__ __forceinline__ void stv(S* p, const float (&o)[4]) {
+  if (V == 4) st4<S>(p, o);
+  else stf<S>(p, o[0]);
+}
+
 // Block-wide sum of up to N values per thread (256 threads); every thread
 // gets the totals.  red must hold N*4 floats.
 template <int N>
@@ -59,7 +94,7 @@ __global__ void __launch_bounds__(256) add_rows_kernel(
 }
 
 // a = norm(x)(1+w1), b = norm(x)(1+w2), s = a + (a_prev - a)*shift.
-template <typename S>
+template <typename S, int V>
 __global__ void __launch_bounds__(256) dual_norm_shift_kernel(
     S* __restrict__ a_out, S* __restrict__ s_out, S* __restrict__ b_out,
     float* __restrict__ last, const float* __restrict__ x,
@@ -79,12 +114,15 @@ __global__ void __launch_bounds__(256) dual_norm_shift_kernel(
   const float* xp = xr - W;  // previous row, only touched when !first
   const bool need_prev_row = shift && !first;
   float ss[2] = {0.f, 0.f};
-  for (int i = threadIdx.x; i < W; i += 256) {
-    const float v = xr[i];
-    ss[0] += v * v;
+  for (int i = threadIdx.x * V; i < W; i += 256 * V) {
+    float xv[4], pv4[4];
+    ldv<float, V>(xr + i, xv);
+#pragma unroll
+    for (int j = 0; j < V; ++j) ss[0] += xv[j] * xv[j];
     if (need_prev_row) {
-      const float p = xp[i];
-      ss[1] += p * p;
+      ldv<float, V>(xp + i, pv4);
+#pragma unroll
+      for (int j = 0; j < V; ++j) ss[1] += pv4[j] * pv4[j];
     }
   }
   block_sum<2>(ss, red);
@@ -92,18 +130,33 @@ __global__ void __launch_bounds__(256) dual_norm_shift_kernel(
   const float rp = 1.0f / sqrtf(ss[1] / (float)W + eps);
   const float* pv = (shift && first && pos > 0)
                         ? prev + (size_t)sslot[b] * W : nullptr;
-  for (int i = threadIdx.x; i < W; i += 256) {
-    const float xv = xr[i];
-    const float g1 = 1.0f + ldf<S>(w1 + i);
-    const float a = xv * r * g1;
-    stf<S>(a_out + (size_t)t * W + i, a);
-    if (b_out) stf<S>(b_out + (size_t)t * W + i, xv * r * (1.0f + ldf<S>(w2 + i)));
+  for (int i = threadIdx.x * V; i < W; i += 256 * V) {
+    float xv[4], g1[4], a[4], o[4], tmp[4];
+    ldv<float, V>(xr + i, xv);
+    ldv<S, V>(w1 + i, g1);
+#pragma unroll
+    for (int j = 0; j < V; ++j) { g1[j] += 1.0f; a[j] = xv[j] * r * g1[j]; }
+    stv<S, V>(a_out + (size_t)t * W + i, a);
+    if (b_out) {
+      ldv<S, V>(w2 + i, tmp);
+#pragma unroll
+      for (int j = 0; j < V; ++j) o[j] = xv[j] * r * (1.0f + tmp[j]);
+      stv<S, V>(b_out + (size_t)t * W + i, o);
+    }
     if (shift) {
-      float ap = 0.f;
-      if (need_prev_row) ap = xp[i] * rp * g1;
-      else if (pv) ap = pv[i];
-      stf<S>(s_out + (size_t)t * W + i, a + (ap - a) * ldf<S>(shift + i));
-      if (is_last) last[(size_t)b * W + i] = a;
+      float ap[4] = {0.f, 0.f, 0.f, 0.f};
+      if (need_prev_row) {
+        ldv<float, V>(xp + i, tmp);
+#pragma unroll
+        for (int j = 0; j < V; ++j) ap[j] = tmp[j] * rp * g1[j];
+      } else if (pv) {
+        ldv<float, V>(pv + i, ap);
+      }
+      ldv<S, V>(shift + i, tmp);
+#pragma unroll
+      for (int j = 0; j < V; ++j) o[j] = a[j] + (ap[j] - a[j]) * tmp[j];
+      stv<S, V>(s_out + (size_t)t * W + i, o);
+      if (is_last) stv<float, V>(last + (size_t)b * W + i, a);
     }
   }
 }
@@ -158,7 +211,7 @@ __global__ void __launch_bounds__(256) headnorm_gate_kernel(
   }
 }
 
-template <typename S>
+template <typename S, int V>
 __global__ void __launch_bounds__(256) polynorm_kernel(
     S* __restrict__ out, const S* __restrict__ z, const float* __restrict__ coef,
     float eps, int F, i64 ldz) {
@@ -166,27 +219,35 @@ __global__ void __launch_bounds__(256) polynorm_kernel(
   const int t = blockIdx.x;
   const S* zr = z + (size_t)t * ldz;
   float s[3] = {0.f, 0.f, 0.f};
-  for (int i = threadIdx.x; i < F; i += 256) {
-    const float v = ldf<S>(zr + i);
-    const float v2 = v * v;
-    s[0] += v2;
-    s[1] += v2 * v2;
-    s[2] += v2 * v2 * v2;
+  for (int i = threadIdx.x * V; i < F; i += 256 * V) {
+    float v[4];
+    ldv<S, V>(zr + i, v);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const float v2 = v[j] * v[j];
+      s[0] += v2;
+      s[1] += v2 * v2;
+      s[2] += v2 * v2 * v2;
+    }
   }
   block_sum<3>(s, red);
   const float r1 = 1.0f / sqrtf(s[0] / (float)F + eps);
   const float r2 = 1.0f / sqrtf(s[1] / (float)F + eps);
   const float r3 = 1.0f / sqrtf(s[2] / (float)F + eps);
   const float c0 = coef[0], c1 = coef[1], c2 = coef[2], c3 = coef[3];
-  for (int i = threadIdx.x; i < F; i += 256) {
-    const float v = ldf<S>(zr + i);
-    const float v2 = v * v;
-    stf<S>(out + (size_t)t * F + i,
-           c0 * (v * r1) + c1 * (v2 * r2) + c2 * (v2 * v * r3) + c3);
+  for (int i = threadIdx.x * V; i < F; i += 256 * V) {
+    float v[4], o[4];
+    ldv<S, V>(zr + i, v);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const float v2 = v[j] * v[j];
+      o[j] = c0 * (v[j] * r1) + c1 * (v2 * r2) + c2 * (v2 * v[j] * r3) + c3;
+    }
+    stv<S, V>(out + (size_t)t * F + i, o);
   }
 }
 
-template <typename S>
+template <typename S, int V>
 __global__ void __launch_bounds__(256) gated_residual_kernel(
     float* __restrict__ x, const S* __restrict__ a, float sa,
     const S* __restrict__ b, float sb, const S* __restrict__ g1, i64 ldg1,
@@ -194,18 +255,27 @@ __global__ void __launch_bounds__(256) gated_residual_kernel(
     const S* __restrict__ g2, i64 ldg2, const float* __restrict__ b2,
     int T, int W) {
   const i64 n = (i64)T * W;
-  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n;
-       i += (i64)gridDim.x * 256) {
+  for (i64 i = ((i64)blockIdx.x * 256 + threadIdx.x) * V; i < n;
+       i += (i64)gridDim.x * 256 * V) {
     const int t = (int)(i / W), c = (int)(i % W);
-    float mix = sa * ldf<S>(a + i);
-    if (b) mix += sb * ldf<S>(b + i);
-    const float z1 = ldf<S>(g1 + (size_t)t * ldg1 + c) + b1[c];
-    float add = mix / (1.0f + expf(-z1));
+    float xv[4], av[4], bv[4] = {0.f, 0.f, 0.f, 0.f}, gv[4], bias[4], mv[4];
+    ldv<float, V>(x + i, xv);
+    ldv<S, V>(a + i, av);
+    if (b) ldv<S, V>(b + i, bv);
+    ldv<S, V>(g1 + (size_t)t * ldg1 + c, gv);
+    ldv<float, V>(b1 + c, bias);
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+      xv[j] += (sa * av[j] + sb * bv[j]) / (1.0f + expf(-(gv[j] + bias[j])));
     if (m) {
-      const float z2 = ldf<S>(g2 + (size_t)t * ldg2 + c) + b2[c];
-      add += ldf<S>(m + i) / (1.0f + expf(-z2));
+      ldv<S, V>(m + i, mv);
+      ldv<S, V>(g2 + (size_t)t * ldg2 + c, gv);
+      ldv<float, V>(b2 + c, bias);
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        xv[j] += mv[j] / (1.0f + expf(-(gv[j] + bias[j])));
     }
-    x[i] += add;
+    stv<float, V>(x + i, xv);
   }
 }
 
@@ -217,6 +287,11 @@ __global__ void __launch_bounds__(256) softcap_kernel(
     const float v = ldf<S>(in + i);
     out[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
   }
+}
+
+template <typename... P>
+inline bool aligned16(P... p) {
+  return ((((uintptr_t)p) % 16 == 0) && ...);
 }
 
 inline int grid_for(i64 n) {
@@ -263,17 +338,16 @@ AF_EXPORT int afm_dual_norm_shift(
   if (shift && (!prev || !last)) return 9003;
   if ((b == nullptr) != (w2 == nullptr)) return 9003;
   hipStream_t s = (hipStream_t)stream;
-  MIX_DISPATCH(dt,
-      (dual_norm_shift_kernel<u16><<<T, 256, 0, s>>>((u16*)a, (u16*)s_out,
-          (u16*)b, (float*)last, (const float*)x, (const u16*)w1,
-          (const u16*)w2, (const u16*)shift, (const float*)prev,
-          (const i32*)row_seq, (const i32*)cu, (const i32*)q_start,
-          (const i32*)sslot, eps, W)),
-      (dual_norm_shift_kernel<float><<<T, 256, 0, s>>>((float*)a,
-          (float*)s_out, (float*)b, (float*)last, (const float*)x,
-          (const float*)w1, (const float*)w2, (const float*)shift,
-          (const float*)prev, (const i32*)row_seq, (const i32*)cu,
-          (const i32*)q_start, (const i32*)sslot, eps, W)));
+  const bool vec = W % 4 == 0 && aligned16(a, s_out, b, last, x, w1) &&
+                   aligned16(w2, shift, prev);
+#define DNS(ST, V)                                                            \
+  dual_norm_shift_kernel<ST, V><<<T, 256, 0, s>>>((ST*)a, (ST*)s_out, (ST*)b, \
+      (float*)last, (const float*)x, (const ST*)w1, (const ST*)w2,            \
+      (const ST*)shift, (const float*)prev, (const i32*)row_seq,              \
+      (const i32*)cu, (const i32*)q_start, (const i32*)sslot, eps, W)
+  if (vec) MIX_DISPATCH(dt, (DNS(u16, 4)), (DNS(float, 4)));
+  else MIX_DISPATCH(dt, (DNS(u16, 1)), (DNS(float, 1)));
+#undef DNS
   return af_last_err();
 }
 
@@ -320,11 +394,13 @@ AF_EXPORT int afm_polynorm(void* out, const void* z, const void* coef,
                            void* stream) {
   if (T == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  MIX_DISPATCH(dt,
-      (polynorm_kernel<u16><<<T, 256, 0, s>>>((u16*)out, (const u16*)z,
-          (const float*)coef, eps, F, ldz)),
-      (polynorm_kernel<float><<<T, 256, 0, s>>>((float*)out, (const float*)z,
-          (const float*)coef, eps, F, ldz)));
+  const bool vec = F % 4 == 0 && ldz % 4 == 0 && aligned16(out, z);
+#define PN(ST, V)                                                     \
+  polynorm_kernel<ST, V><<<T, 256, 0, s>>>((ST*)out, (const ST*)z,    \
+      (const float*)coef, eps, F, ldz)
+  if (vec) MIX_DISPATCH(dt, (PN(u16, 4)), (PN(float, 4)));
+  else MIX_DISPATCH(dt, (PN(u16, 1)), (PN(float, 1)));
+#undef PN
   return af_last_err();
 }
 
@@ -335,16 +411,17 @@ AF_EXPORT int afm_gated_residual(
   if (T == 0) return 0;
   if (m && (!g2 || !b2)) return 9003;
   hipStream_t s = (hipStream_t)stream;
-  const int grid = grid_for((i64)T * W);
-  MIX_DISPATCH(dt,
-      (gated_residual_kernel<u16><<<grid, 256, 0, s>>>((float*)x,
-          (const u16*)a, sa, (const u16*)b, sb, (const u16*)g1, ldg1,
-          (const float*)b1, (const u16*)m, (const u16*)g2, ldg2,
-          (const float*)b2, T, W)),
-      (gated_residual_kernel<float><<<grid, 256, 0, s>>>((float*)x,
-          (const float*)a, sa, (const float*)b, sb, (const float*)g1, ldg1,
-          (const float*)b1, (const float*)m, (const float*)g2, ldg2,
-          (const float*)b2, T, W)));
+  const bool vec = W % 4 == 0 && ldg1 % 4 == 0 && ldg2 % 4 == 0 &&
+                   aligned16(x, a, b, g1, b1, m) && aligned16(g2, b2);
+  const int grid = grid_for((i64)T * W / (vec ? 4 : 1));
+#define GR(ST, V)                                                          \
+  gated_residual_kernel<ST, V><<<grid, 256, 0, s>>>((float*)x,             \
+      (const ST*)a, sa, (const ST*)b, sb, (const ST*)g1, ldg1,             \
+      (const float*)b1, (const ST*)m, (const ST*)g2, ldg2, (const float*)b2, \
+      T, W)
+  if (vec) MIX_DISPATCH(dt, (GR(u16, 4)), (GR(float, 4)));
+  else MIX_DISPATCH(dt, (GR(u16, 1)), (GR(float, 1)));
+#undef GR
   return af_last_err();
 }
 

@@ -177,61 +177,99 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
   }
   const float hd = head_decay ? head_decay[h] : 1.0f;
   const int half = rot >> 1;
-  for (int tb = t0; tb < t1; tb += SCAN_TB) {
+  // raw operands of the next block, fetched while the current one computes
+  constexpr int EPT = SCAN_TB * DKP / 256;   // staged elements per thread
+  float rq[EPT], rk[EPT], rqp[EPT], rkp[EPT], rz[EPT], rpos[EPT];
+  float rv[(SCAN_TB * 32 + 255) / 256];
+  auto fetch = [&](int tb) {
     const int nt = min(SCAN_TB, t1 - tb);
-    // ---- stage nt tokens: q, k (rotated, scaled) and decay rows ----
-    for (int e = threadIdx.x; e < nt * DKP; e += 256) {
+#pragma unroll
+    for (int n = 0; n < EPT; ++n) {
+      const int e = threadIdx.x + 256 * n;
       const int tt = e / DKP, i = e % DKP;
-      float* row = stage + (size_t)tt * 3 * DKP;
-      float qv = 0.f, kv = 0.f, a = 0.f;
-      if (i < dk) {
+      rq[n] = rk[n] = rqp[n] = rkp[n] = rz[n] = rpos[n] = 0.f;
+      if (tt < nt && i < dk) {
         const int t = tb + tt;
         const S* qr = q + (size_t)t * ldq + (size_t)h * dk;
         const S* kr = k + (size_t)t * ldk + (size_t)h * dk;
-        qv = ldf<S>(qr + i);
-        kv = ldf<S>(kr + i);
+        rq[n] = ldf<S>(qr + i);
+        rk[n] = ldf<S>(kr + i);
+        if (i < rot) {
+          const int pi = i < half ? i + half : i - half;
+          rqp[n] = ldf<S>(qr + pi);
+          rkp[n] = ldf<S>(kr + pi);
+          rpos[n] = (float)positions[t];
+        }
+        if (zl) rz[n] = ldf<S>(zl + (size_t)t * ldz + (size_t)h * dk + i);
+      }
+    }
+#pragma unroll
+    for (int n = 0; n < (SCAN_TB * 32 + 255) / 256; ++n) {
+      const int e = threadIdx.x + 256 * n;
+      const int tt = e >> 5, ci = c0 + (e & 31);
+      rv[n] = (tt < nt && ci < dv)
+                  ? ldf<S>(v + (size_t)(tb + tt) * ldv + (size_t)h * dv + ci) : 0.f;
+    }
+  };
+  fetch(t0);
+  for (int tb = t0; tb < t1; tb += SCAN_TB) {
+    const int nt = min(SCAN_TB, t1 - tb);
+    // ---- stage the block: rotate / scale q, k; evaluate the decays ----
+#pragma unroll
+    for (int n = 0; n < EPT; ++n) {
+      const int e = threadIdx.x + 256 * n;
+      const int tt = e / DKP, i = e % DKP;
+      float* row = stage + (size_t)tt * 3 * DKP;
+      float qv = rq[n], kv = rk[n], a = 0.f;
+      if (tt < nt && i < dk) {
         if (i < rot) {
           const bool lowh = i < half;
-          const int fi = lowh ? i : i - half;
-          const int pi = lowh ? i + half : i - half;
-          const float ang = (float)positions[t] * inv_freq[fi];
-          const float cs = cosf(ang), sn = sinf(ang);
-          const float qp = ldf<S>(qr + pi), kp = ldf<S>(kr + pi);
+          float sn, cs;
+          sincosf(rpos[n] * inv_freq[lowh ? i : i - half], &sn, &cs);
           // pair (u, w) -> (u cos - w sin, w cos + u sin)
-          qv = lowh ? qv * cs - qp * sn : qv * cs + qp * sn;
-          kv = lowh ? kv * cs - kp * sn : kv * cs + kp * sn;
+          qv = lowh ? qv * cs - rqp[n] * sn : qv * cs + rqp[n] * sn;
+          kv = lowh ? kv * cs - rkp[n] * sn : kv * cs + rkp[n] * sn;
         }
         qv *= q_scale;
         kv *= k_scale;
         a = hd;
         if (zl) {
-          const float z = ldf<S>(zl + (size_t)t * ldz + (size_t)h * dk + i) +
-                          zbias[(size_t)h * dk + i];
+          const float z = rz[n] + zbias[(size_t)h * dk + i];
           // log(sigmoid(z)) = -softplus(-z), evaluated without overflow
           const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
           a = expf(ls * inv_tau);
         }
       }
-      row[i] = qv;
-      row[DKP + i] = kv;
-      row[2 * DKP + i] = a;
+      if (tt < SCAN_TB) {
+        row[i] = qv;
+        row[DKP + i] = kv;
+        row[2 * DKP + i] = a;
+      }
     }
-    for (int e = threadIdx.x; e < nt * 32; e += 256) {
-      const int tt = e >> 5, ci = c0 + (e & 31);
-      vs[e] = ci < dv ? ldf<S>(v + (size_t)(tb + tt) * ldv + (size_t)h * dv + ci) : 0.f;
+#pragma unroll
+    for (int n = 0; n < (SCAN_TB * 32 + 255) / 256; ++n) {
+      const int e = threadIdx.x + 256 * n;
+      if (e < SCAN_TB * 32) vs[e] = rv[n];
     }
     __syncthreads();
+    if (tb + SCAN_TB < t1) fetch(tb + SCAN_TB);   // in flight during compute
     // ---- advance this thread's rows through the block, token by token ----
     for (int tt = 0; tt < nt; ++tt) {
-      const float* sq = stage + (size_t)tt * 3 * DKP + r * RP;
-      const float* sk = sq + DKP;
-      const float* sa = sk + DKP;
+      const f32x4* sq = reinterpret_cast<const f32x4*>(
+          stage + (size_t)tt * 3 * DKP + r * RP);
+      const f32x4* sk = sq + DKP / 4;
+      const f32x4* sa = sk + DKP / 4;
       const float vv = vs[tt * 32 + cc];
       float p = 0.f;
 #pragma unroll
-      for (int ii = 0; ii < RP; ++ii) {
-        st[ii] = sa[ii] * st[ii] + sk[ii] * vv;
-        p += st[ii] * sq[ii];
+      for (int i4 = 0; i4 < RP / 4; ++i4) {
+        const f32x4 a4 = sa[i4], k4 = sk[i4], q4 = sq[i4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int ii = i4 * 4 + j;
+          st[ii] = a4[j] * st[ii] + k4[j] * vv;
+          p += st[ii] * q4[j];
+        }
       }
       part[tt * 256 + r * 32 + cc] = p;
     }
