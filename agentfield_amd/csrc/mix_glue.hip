@@ -189,7 +189,7 @@ __global__ void __launch_bounds__(256) norm_rows_kernel(
 }
 
 // One wave per (row, head): RMS over dv of fp32 o, * weight, * silu(gate).
-template <typename S>
+template <typename S, int V>
 __global__ void __launch_bounds__(256) headnorm_gate_kernel(
     S* __restrict__ out, const float* __restrict__ o, const S* __restrict__ g,
     const S* __restrict__ w, float eps, int n_rh, int H, int dv, i64 ldg) {
@@ -199,15 +199,24 @@ __global__ void __launch_bounds__(256) headnorm_gate_kernel(
   const int t = rh / H, h = rh % H;
   const float* orow = o + ((size_t)t * H + h) * dv;
   float ss = 0.f;
-  for (int d = lane; d < dv; d += 64) ss += orow[d] * orow[d];
+  for (int d = lane * V; d < dv; d += 64 * V) {
+    float ov[4];
+    ldv<float, V>(orow + d, ov);
+#pragma unroll
+    for (int j = 0; j < V; ++j) ss += ov[j] * ov[j];
+  }
   ss = wave_sum_f32(ss);
   const float rs = 1.0f / sqrtf(ss / (float)dv + eps);
   const S* grow = g + (size_t)t * ldg + (size_t)h * dv;
-  for (int d = lane; d < dv; d += 64) {
-    const float gv = ldf<S>(grow + d);
-    float v = orow[d] * rs;
-    if (w) v *= ldf<S>(w + d);
-    stf<S>(out + ((size_t)t * H + h) * dv + d, v * (gv / (1.0f + expf(-gv))));
+  for (int d = lane * V; d < dv; d += 64 * V) {
+    float ov[4], gv[4], wv[4] = {1.f, 1.f, 1.f, 1.f}, r[4];
+    ldv<float, V>(orow + d, ov);
+    ldv<S, V>(grow + d, gv);
+    if (w) ldv<S, V>(w + d, wv);
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+      r[j] = ov[j] * rs * wv[j] * (gv[j] / (1.0f + expf(-gv[j])));
+    stv<S, V>(out + ((size_t)t * H + h) * dv + d, r);
   }
 }
 
@@ -380,12 +389,13 @@ AF_EXPORT int afm_headnorm_gate(void* out, const void* o, const void* g,
   const int n_rh = T * H;
   const int grid = (n_rh + 3) / 4;
   hipStream_t s = (hipStream_t)stream;
-  MIX_DISPATCH(dt,
-      (headnorm_gate_kernel<u16><<<grid, 256, 0, s>>>((u16*)out,
-          (const float*)o, (const u16*)g, (const u16*)w, eps, n_rh, H, dv, ldg)),
-      (headnorm_gate_kernel<float><<<grid, 256, 0, s>>>((float*)out,
-          (const float*)o, (const float*)g, (const float*)w, eps, n_rh, H, dv,
-          ldg)));
+  const bool vec = dv % 4 == 0 && ldg % 4 == 0 && aligned16(out, o, g, w);
+#define HG(ST, V)                                                           \
+  headnorm_gate_kernel<ST, V><<<grid, 256, 0, s>>>((ST*)out, (const float*)o, \
+      (const ST*)g, (const ST*)w, eps, n_rh, H, dv, ldg)
+  if (vec) MIX_DISPATCH(dt, (HG(u16, 4)), (HG(float, 4)));
+  else MIX_DISPATCH(dt, (HG(u16, 1)), (HG(float, 1)));
+#undef HG
   return af_last_err();
 }
 

@@ -18,8 +18,44 @@ template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p =
 
 // ---------------------------------------------------------------- qk norm
 // One workgroup per row.  q row [nq], k row [nk], v row [nv]; caches
-// [P, G, page, dk|dv]; slot = page_index*page + offset.
-template <typename S>
+// [P, G, page, dk|dv]; slot = page_index*page + offset.  V = 4: 4-element
+// vector accesses (sizes and strides multiples of 4), V = 1: scalar.
+template <typename S, int V>
+__device__ __forceinline__ void ldvs(const S* p, float (&o)[4]) {
+  if (V == 4) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = 0.f;
+    if constexpr (sizeof(S) == 2) {
+      const s16x4 v = *reinterpret_cast<const s16x4*>(p);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = bf2f((u16)v[j]);
+    } else {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(p);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = v[j];
+    }
+  } else {
+    o[0] = ldf<S>(p);
+    o[1] = o[2] = o[3] = 0.f;
+  }
+}
+template <typename S, int V>
+__device__ __forceinline__ void stvs(S* p, const float (&o)[4]) {
+  if (V == 4) {
+    if constexpr (sizeof(S) == 2) {
+      s16x4 v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = (short)f2bf(o[j]);
+      *reinterpret_cast<s16x4*>(p) = v;
+    } else {
+      *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+    }
+  } else {
+    stf<S>(p, o[0]);
+  }
+}
+
+template <typename S, int V>
 __global__ void __launch_bounds__(256) qk_norm_cache_kernel(
     S* __restrict__ qout, const S* __restrict__ q, const S* __restrict__ k,
     const S* __restrict__ v, const S* __restrict__ qw, const S* __restrict__ kw,
@@ -32,8 +68,17 @@ __global__ void __launch_bounds__(256) qk_norm_cache_kernel(
   const S* kr = k + (size_t)t * ldk;
   const S* vr = v + (size_t)t * ldv;
   float sq = 0.f, sk = 0.f;
-  for (int i = threadIdx.x; i < nq; i += 256) { const float f = ldf<S>(qr + i); sq += f * f; }
-  for (int i = threadIdx.x; i < nk; i += 256) { const float f = ldf<S>(kr + i); sk += f * f; }
+  float f[4], w4[4];
+  for (int i = threadIdx.x * V; i < nq; i += 256 * V) {
+    ldvs<S, V>(qr + i, f);
+#pragma unroll
+    for (int j = 0; j < V; ++j) sq += f[j] * f[j];
+  }
+  for (int i = threadIdx.x * V; i < nk; i += 256 * V) {
+    ldvs<S, V>(kr + i, f);
+#pragma unroll
+    for (int j = 0; j < V; ++j) sk += f[j] * f[j];
+  }
   sq = wave_sum_f32(sq);
   sk = wave_sum_f32(sk);
   if ((threadIdx.x & 63) == 0) {
@@ -43,23 +88,32 @@ __global__ void __launch_bounds__(256) qk_norm_cache_kernel(
   __syncthreads();
   const float rq = qw ? 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)nq + eps) : 1.0f;
   const float rk = kw ? 1.0f / sqrtf((red[4] + red[5] + red[6] + red[7]) / (float)nk + eps) : 1.0f;
-  for (int i = threadIdx.x; i < nq; i += 256) {
-    float f = ldf<S>(qr + i) * rq;
-    if (qw) f *= ldf<S>(qw + i);
-    stf<S>(qout + (size_t)t * nq + i, f);
+  for (int i = threadIdx.x * V; i < nq; i += 256 * V) {
+    ldvs<S, V>(qr + i, f);
+    if (qw) {
+      ldvs<S, V>(qw + i, w4);
+#pragma unroll
+      for (int j = 0; j < V; ++j) f[j] *= rq * w4[j];
+    }
+    stvs<S, V>(qout + (size_t)t * nq + i, f);
   }
   const i64 sl = slots[t];
   if (sl < 0) return;
   const i64 pg = sl / page, off = sl % page;
-  for (int i = threadIdx.x; i < nk; i += 256) {
+  for (int i = threadIdx.x * V; i < nk; i += 256 * V) {
     const int g = i / dk, d = i % dk;
-    float f = ldf<S>(kr + i) * rk;
-    if (kw) f *= ldf<S>(kw + i);
-    stf<S>(kc + (((size_t)pg * G + g) * page + off) * dk + d, f);
+    ldvs<S, V>(kr + i, f);
+    if (kw) {
+      ldvs<S, V>(kw + i, w4);
+#pragma unroll
+      for (int j = 0; j < V; ++j) f[j] *= rk * w4[j];
+    }
+    stvs<S, V>(kc + (((size_t)pg * G + g) * page + off) * dk + d, f);
   }
-  for (int i = threadIdx.x; i < nv; i += 256) {
+  for (int i = threadIdx.x * V; i < nv; i += 256 * V) {
     const int g = i / dv, d = i % dv;
-    vc[(((size_t)pg * G + g) * page + off) * dv + d] = vr[i];
+    ldvs<S, V>(vr + i, f);
+    stvs<S, V>(vc + (((size_t)pg * G + g) * page + off) * dv + d, f);
   }
 }
 
@@ -307,18 +361,19 @@ AF_EXPORT int afm_qk_norm_cache(
   if (T == 0) return 0;
   if (nk != G * dk || nv != G * dv) return 9003;
   hipStream_t s = (hipStream_t)stream;
-  if (dt == 0)
-    qk_norm_cache_kernel<u16><<<T, 256, 0, s>>>((u16*)qout, (const u16*)q,
-        (const u16*)k, (const u16*)v, (const u16*)qw, (const u16*)kw, (u16*)kc,
-        (u16*)vc, (const i64*)slots, eps, nq, nk, nv, G, dk, dv, page, ldq,
-        ldk, ldv);
-  else if (dt == 1)
-    qk_norm_cache_kernel<float><<<T, 256, 0, s>>>((float*)qout,
-        (const float*)q, (const float*)k, (const float*)v, (const float*)qw,
-        (const float*)kw, (float*)kc, (float*)vc, (const i64*)slots, eps, nq,
-        nk, nv, G, dk, dv, page, ldq, ldk, ldv);
-  else
-    return 9002;
+  auto al = [](const void* p) { return p == nullptr || (uintptr_t)p % 16 == 0; };
+  const bool vec = dk % 4 == 0 && dv % 4 == 0 && nq % 4 == 0 && ldq % 4 == 0 &&
+                   ldk % 4 == 0 && ldv % 4 == 0 && al(qout) && al(q) && al(k) &&
+                   al(v) && al(qw) && al(kw) && al(kc) && al(vc);
+#define QKN(ST, V)                                                            \
+  qk_norm_cache_kernel<ST, V><<<T, 256, 0, s>>>((ST*)qout, (const ST*)q,      \
+      (const ST*)k, (const ST*)v, (const ST*)qw, (const ST*)kw, (ST*)kc,      \
+      (ST*)vc, (const i64*)slots, eps, nq, nk, nv, G, dk, dv, page, ldq, ldk, \
+      ldv)
+  if (dt == 0) { if (vec) QKN(u16, 4); else QKN(u16, 1); }
+  else if (dt == 1) { if (vec) QKN(float, 4); else QKN(float, 1); }
+  else return 9002;
+#undef QKN
   return af_last_err();
 }
 
