@@ -189,13 +189,14 @@ __global__ void __launch_bounds__(256) masked_attention_kernel(
 }
 
 // ------------------------------------------------------------- linear scan
-// Workgroup = (sequence, head, 32-column tile of dv); 256 threads = 8 row
-// groups x 32 columns.  Thread (r, c) keeps RP consecutive rows
-// r*RP .. r*RP+RP-1 of column c of the state in registers.  Tokens are
+// Workgroup = (sequence, head, 32-column tile of dv); 256 threads = 16 row
+// groups x 16 column pairs.  Thread (r, c) keeps RP consecutive rows
+// r*RP .. r*RP+RP-1 of columns c and c+16 of the state in registers (each
+// q / k / decay value read from LDS feeds two columns).  Tokens are
 // walked serially in blocks of TB: the block's q / k / decay rows are staged
 // into LDS at once (rotary + scaling applied on the way in), every thread
 // then advances its rows through the TB tokens without synchronising and
-// leaves one partial output per token in LDS, and the 8 partials of each
+// leaves one partial output per token in LDS, and the 16 partials of each
 // (token, column) are summed after one more barrier: two barriers per TB
 // tokens, the recurrence itself strictly token by token in fp32 — so results
 // are bit-identical however a sequence is cut into chunks.
@@ -209,25 +210,29 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
     const i32* __restrict__ q_start, const i32* __restrict__ sslot,
     float q_scale, float k_scale, float inv_tau, int H, int dk, int dv,
     int rot, i64 ldq, i64 ldk, i64 ldv, i64 ldz) {
-  constexpr int DKP = 8 * RP;          // padded rows: zeros beyond dk
-  constexpr int SCAN_TB = RP >= 32 ? 8 : 16;  // keeps LDS under 64 KB
-  extern __shared__ float smem[];      // [TB][3][DKP] + [TB][8][32] + [TB][32]
+  constexpr int DKP = 16 * RP;         // padded rows: zeros beyond dk
+  // bf16 operands carry 2^-9 relative rounding already: hardware
+  // transcendentals there; fp32 storage keeps the precise library forms
+  constexpr bool FAST = sizeof(S) == 2;
+  constexpr int SCAN_TB = RP >= 16 ? 8 : 16;  // keeps LDS under 64 KB
+  extern __shared__ float smem[];      // [TB][3][DKP] + [TB][16][32] + [TB][32]
   const int b = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 32;
   const int t0 = cu[b], t1 = cu[b + 1];
   if (t1 <= t0) return;
-  const int r = threadIdx.x >> 5, cc = threadIdx.x & 31;
-  const int c = c0 + cc;
-  const bool cok = c < dv;
+  const int r = threadIdx.x >> 4, cc = threadIdx.x & 15;
+  const int ca = c0 + cc, cb = c0 + cc + 16;
+  const bool oka = ca < dv, okb = cb < dv;
   float* stage = smem;                         // [TB][3][DKP]: q, k, decay
-  float* part = smem + SCAN_TB * 3 * DKP;      // [TB][8][32]
-  float* vs = part + SCAN_TB * 256;            // [TB][32]
+  float* part = smem + SCAN_TB * 3 * DKP;      // [TB][16][32]
+  float* vs = part + SCAN_TB * 512;            // [TB][32]
   float* sbase = state + (((size_t)sslot[b] * H + h) * dk) * dv;
-  float st[RP];
+  float sta[RP], stb[RP];
   const bool fresh = q_start[b] == 0;
 #pragma unroll
   for (int ii = 0; ii < RP; ++ii) {
     const int i = r * RP + ii;
-    st[ii] = (!fresh && cok && i < dk) ? sbase[(size_t)i * dv + c] : 0.f;
+    sta[ii] = (!fresh && oka && i < dk) ? sbase[(size_t)i * dv + ca] : 0.f;
+    stb[ii] = (!fresh && okb && i < dk) ? sbase[(size_t)i * dv + cb] : 0.f;
   }
   const float hd = head_decay ? head_decay[h] : 1.0f;
   const int half = rot >> 1;
@@ -235,34 +240,51 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
   constexpr int EPT = SCAN_TB * DKP / 256;   // staged elements per thread
   float rq[EPT], rk[EPT], rqp[EPT], rkp[EPT], rz[EPT], rpos[EPT];
   float rv[(SCAN_TB * 32 + 255) / 256];
+  // Every load is unconditional on a clamped address (invalid lanes are
+  // zeroed afterwards), so all of a block's loads are in flight together
+  // instead of one exposed memory latency per guarded element.
   auto fetch = [&](int tb) {
     const int nt = min(SCAN_TB, t1 - tb);
 #pragma unroll
     for (int n = 0; n < EPT; ++n) {
       const int e = threadIdx.x + 256 * n;
       const int tt = e / DKP, i = e % DKP;
-      rq[n] = rk[n] = rqp[n] = rkp[n] = rz[n] = rpos[n] = 0.f;
-      if (tt < nt && i < dk) {
-        const int t = tb + tt;
-        const S* qr = q + (size_t)t * ldq + (size_t)h * dk;
-        const S* kr = k + (size_t)t * ldk + (size_t)h * dk;
-        rq[n] = ldf<S>(qr + i);
-        rk[n] = ldf<S>(kr + i);
-        if (i < rot) {
-          const int pi = i < half ? i + half : i - half;
-          rqp[n] = ldf<S>(qr + pi);
-          rkp[n] = ldf<S>(kr + pi);
-          rpos[n] = (float)positions[t];
-        }
-        if (zl) rz[n] = ldf<S>(zl + (size_t)t * ldz + (size_t)h * dk + i);
+      const bool valid = tt < nt && i < dk;
+      const int t = tb + min(tt, nt - 1), ic = min(i, dk - 1);
+      const float a = ldf<S>(q + (size_t)t * ldq + (size_t)h * dk + ic);
+      const float c = ldf<S>(k + (size_t)t * ldk + (size_t)h * dk + ic);
+      rq[n] = valid ? a : 0.f;
+      rk[n] = valid ? c : 0.f;
+      rqp[n] = rkp[n] = rz[n] = rpos[n] = 0.f;
+    }
+    if (rot > 0) {
+#pragma unroll
+      for (int n = 0; n < EPT; ++n) {
+        const int e = threadIdx.x + 256 * n;
+        const int tt = e / DKP, i = e % DKP;
+        const int t = tb + min(tt, nt - 1), ic = min(i, dk - 1);
+        const int pi = ic < half ? ic + half : (ic < rot ? ic - half : ic);
+        rqp[n] = ldf<S>(q + (size_t)t * ldq + (size_t)h * dk + pi);
+        rkp[n] = ldf<S>(k + (size_t)t * ldk + (size_t)h * dk + pi);
+        rpos[n] = (float)positions[t];
+      }
+    }
+    if (zl) {
+#pragma unroll
+      for (int n = 0; n < EPT; ++n) {
+        const int e = threadIdx.x + 256 * n;
+        const int tt = e / DKP, i = e % DKP;
+        const int t = tb + min(tt, nt - 1), ic = min(i, dk - 1);
+        rz[n] = ldf<S>(zl + (size_t)t * ldz + (size_t)h * dk + ic);
       }
     }
 #pragma unroll
     for (int n = 0; n < (SCAN_TB * 32 + 255) / 256; ++n) {
       const int e = threadIdx.x + 256 * n;
       const int tt = e >> 5, ci = c0 + (e & 31);
-      rv[n] = (tt < nt && ci < dv)
-                  ? ldf<S>(v + (size_t)(tb + tt) * ldv + (size_t)h * dv + ci) : 0.f;
+      const float x = ldf<S>(v + (size_t)(tb + min(tt, nt - 1)) * ldv +
+                             (size_t)h * dv + min(ci, dv - 1));
+      rv[n] = (tt < nt && ci < dv) ? x : 0.f;
     }
   };
   fetch(t0);
@@ -279,7 +301,9 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
         if (i < rot) {
           const bool lowh = i < half;
           float sn, cs;
-          sincosf(rpos[n] * inv_freq[lowh ? i : i - half], &sn, &cs);
+          const float ang = rpos[n] * inv_freq[lowh ? i : i - half];
+          if (FAST) { sn = __sinf(ang); cs = __cosf(ang); }
+          else sincosf(ang, &sn, &cs);
           // pair (u, w) -> (u cos - w sin, w cos + u sin)
           qv = lowh ? qv * cs - rqp[n] * sn : qv * cs + rqp[n] * sn;
           kv = lowh ? kv * cs - rkp[n] * sn : kv * cs + rkp[n] * sn;
@@ -290,8 +314,14 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
         if (zl) {
           const float z = rz[n] + zbias[(size_t)h * dk + i];
           // log(sigmoid(z)) = -softplus(-z), evaluated without overflow
-          const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
-          a = expf(ls * inv_tau);
+          if (FAST) {
+            const float ls = z >= 0.f ? -__logf(1.0f + __expf(-z))
+                                      : z - __logf(1.0f + __expf(z));
+            a = __expf(ls * inv_tau);
+          } else {
+            const float ls = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
+            a = expf(ls * inv_tau);
+          }
         }
       }
       if (tt < SCAN_TB) {
@@ -308,46 +338,56 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
     __syncthreads();
     if (tb + SCAN_TB < t1) fetch(tb + SCAN_TB);   // in flight during compute
     // ---- advance this thread's rows through the block, token by token ----
-    for (int tt = 0; tt < nt; ++tt) {
-      const f32x4* sq = reinterpret_cast<const f32x4*>(
+    auto step = [&](int tt) {
+      const f32x2* sq = reinterpret_cast<const f32x2*>(
           stage + (size_t)tt * 3 * DKP + r * RP);
-      const f32x4* sk = sq + DKP / 4;
-      const f32x4* sa = sk + DKP / 4;
-      const float vv = vs[tt * 32 + cc];
-      float p = 0.f;
+      const f32x2* sk = sq + DKP / 2;
+      const f32x2* sa = sk + DKP / 2;
+      const float va = vs[tt * 32 + cc], vb = vs[tt * 32 + cc + 16];
+      float pa = 0.f, pb = 0.f;
 #pragma unroll
-      for (int i4 = 0; i4 < RP / 4; ++i4) {
-        const f32x4 a4 = sa[i4], k4 = sk[i4], q4 = sq[i4];
+      for (int i2 = 0; i2 < RP / 2; ++i2) {
+        const f32x2 a2 = sa[i2], k2 = sk[i2], q2 = sq[i2];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int ii = i4 * 4 + j;
-          st[ii] = a4[j] * st[ii] + k4[j] * vv;
-          p += st[ii] * q4[j];
+        for (int j = 0; j < 2; ++j) {
+          const int ii = i2 * 2 + j;
+          sta[ii] = a2[j] * sta[ii] + k2[j] * va;
+          stb[ii] = a2[j] * stb[ii] + k2[j] * vb;
+          pa += sta[ii] * q2[j];
+          pb += stb[ii] * q2[j];
         }
       }
-      part[tt * 256 + r * 32 + cc] = p;
+      part[tt * 512 + r * 32 + cc] = pa;
+      part[tt * 512 + r * 32 + cc + 16] = pb;
+    };
+    if (nt == SCAN_TB) {
+      // full block: fixed trip count, so the LDS reads of later tokens are
+      // scheduled under the arithmetic of earlier ones
+#pragma unroll
+      for (int tt = 0; tt < SCAN_TB; ++tt) step(tt);
+    } else {
+      for (int tt = 0; tt < nt; ++tt) step(tt);
     }
     __syncthreads();
-    // ---- o[t][c] = sum of the 8 row-group partials ----
+    // ---- o[t][c] = sum of the 16 row-group partials ----
     for (int e = threadIdx.x; e < nt * 32; e += 256) {
       const int tt = e >> 5, ci = e & 31;
       if (c0 + ci < dv) {
-        const float* pr = part + tt * 256 + ci;
+        const float* pr = part + tt * 512 + ci;
         float o = 0.f;
 #pragma unroll
-        for (int rr = 0; rr < 8; ++rr) o += pr[rr * 32];
+        for (int rr = 0; rr < 16; ++rr) o += pr[rr * 32];
         out[(size_t)(tb + tt) * H * dv + (size_t)h * dv + c0 + ci] = o;
       }
     }
     // the next block's staging writes `stage`/`vs`, last read before the
     // barrier above; its partials are written after the next barrier
   }
-  if (cok) {
 #pragma unroll
-    for (int ii = 0; ii < RP; ++ii) {
-      const int i = r * RP + ii;
-      if (i < dk) sbase[(size_t)i * dv + c] = st[ii];
-    }
+  for (int ii = 0; ii < RP; ++ii) {
+    const int i = r * RP + ii;
+    if (i < dk && oka) sbase[(size_t)i * dv + ca] = sta[ii];
+    if (i < dk && okb) sbase[(size_t)i * dv + cb] = stb[ii];
   }
 }
 
@@ -426,18 +466,18 @@ static int launch_scan(float* out, float* state, const void* q, const void* k,
                        float inv_tau, int B, int H, int dk, int dv, int rot,
                        i64 ldq, i64 ldk, i64 ldv, i64 ldz, hipStream_t s) {
   dim3 grid(B, H, (dv + 31) / 32);
-  const int rp = (dk + 7) / 8;
-  const int rpp = rp <= 4 ? 4 : rp <= 8 ? 8 : rp <= 16 ? 16 : 32;
-  const size_t sm = (size_t)(rpp >= 32 ? 8 : 16) * (3 * 8 * rpp + 256 + 32) * sizeof(float);
+  const int rp = (dk + 15) / 16;
+  const int rpp = rp <= 2 ? 2 : rp <= 4 ? 4 : rp <= 8 ? 8 : 16;
+  const size_t sm = (size_t)(rpp >= 16 ? 8 : 16) * (3 * 16 * rpp + 512 + 32) * sizeof(float);
 #define SCAN(RP)                                                             \
   linear_scan_kernel<S, RP><<<grid, 256, sm, s>>>(                           \
       out, state, (const S*)q, (const S*)k, (const S*)v, (const S*)zl, zbias, \
       head_decay, inv_freq, positions, cu, q_start, sslot, q_scale, k_scale, \
       inv_tau, H, dk, dv, rot, ldq, ldk, ldv, ldz)
-  if (rp <= 4) SCAN(4);
+  if (rp <= 2) SCAN(2);
+  else if (rp <= 4) SCAN(4);
   else if (rp <= 8) SCAN(8);
-  else if (rp <= 16) SCAN(16);
-  else SCAN(32);
+  else SCAN(16);
 #undef SCAN
   return af_last_err();
 }
