@@ -361,11 +361,15 @@ class LLMEngine:
     def _state_slot(self, seq: Sequence) -> int:
         live = None
         if self.state_slots.num_free == 0:
+            # out of slots: sequences preempted since they got theirs still
+            # own one; everything not running any more gives it back
             running = getattr(self.sched, "running", None)
-            if running is not None:
-                live = {s.seq_id for s in running}
-                live.update(s.seq_id for s in self._prefilling)
-                live.update(self._open)
+            if running is None:   # native adapter keeps a seq_id -> seq map
+                running = [s for s in self.sched.seqs.values()
+                           if s.status == SeqStatus.RUNNING]
+            live = {s.seq_id for s in running}
+            live.update(s.seq_id for s in self._prefilling)
+            live.update(self._open)
         return self.state_slots.slot_of(seq, live)
 
     def _chunk_batch(self, seqs: list[Sequence], starts: list[int],
