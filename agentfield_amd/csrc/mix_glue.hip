@@ -99,10 +99,13 @@ __global__ void __launch_bounds__(256) dual_norm_shift_kernel(
     S* __restrict__ a_out, S* __restrict__ s_out, S* __restrict__ b_out,
     float* __restrict__ last, const float* __restrict__ x,
     const S* __restrict__ w1, const S* __restrict__ w2,
-    const S* __restrict__ shift, const float* __restrict__ prev,
+    const S* __restrict__ shift, float* prev,
     const i32* __restrict__ row_seq, const i32* __restrict__ cu,
     const i32* __restrict__ q_start, const i32* __restrict__ sslot,
     float eps, int W) {
+  // last == nullptr: every chunk is a single row (a decode step); the row's
+  // norm goes straight into its state slot, each element read before it is
+  // overwritten by the same thread.
   __shared__ float red[8];
   const int t = blockIdx.x;
   const int b = row_seq[t];
@@ -156,7 +159,9 @@ __global__ void __launch_bounds__(256) dual_norm_shift_kernel(
 #pragma unroll
       for (int j = 0; j < V; ++j) o[j] = a[j] + (ap[j] - a[j]) * tmp[j];
       stv<S, V>(s_out + (size_t)t * W + i, o);
-      if (is_last) stv<float, V>(last + (size_t)b * W + i, a);
+      if (is_last)
+        stv<float, V>(last ? last + (size_t)b * W + i
+                           : prev + (size_t)sslot[b] * W + i, a);
     }
   }
 }
@@ -344,7 +349,7 @@ AF_EXPORT int afm_dual_norm_shift(
     const void* cu, const void* q_start, const void* sslot, float eps, int T,
     int W, int dt, void* stream) {
   if (T == 0) return 0;
-  if (shift && (!prev || !last)) return 9003;
+  if (shift && !prev) return 9003;
   if ((b == nullptr) != (w2 == nullptr)) return 9003;
   hipStream_t s = (hipStream_t)stream;
   const bool vec = W % 4 == 0 && aligned16(a, s_out, b, last, x, w1) &&
@@ -352,7 +357,7 @@ AF_EXPORT int afm_dual_norm_shift(
 #define DNS(ST, V)                                                            \
   dual_norm_shift_kernel<ST, V><<<T, 256, 0, s>>>((ST*)a, (ST*)s_out, (ST*)b, \
       (float*)last, (const float*)x, (const ST*)w1, (const ST*)w2,            \
-      (const ST*)shift, (const float*)prev, (const i32*)row_seq,              \
+      (const ST*)shift, (float*)prev, (const i32*)row_seq,                    \
       (const i32*)cu, (const i32*)q_start, (const i32*)sslot, eps, W)
   if (vec) MIX_DISPATCH(dt, (DNS(u16, 4)), (DNS(float, 4)));
   else MIX_DISPATCH(dt, (DNS(u16, 1)), (DNS(float, 1)));

@@ -123,8 +123,12 @@ def dual_norm_shift(x: torch.Tensor, w1: torch.Tensor,
     a = torch.empty(T, W, dtype=out_dtype, device=x.device)
     s = torch.empty_like(a) if shift is not None else a
     b = torch.empty_like(a) if w2 is not None else None
+    # a decode step (one row per sequence) writes the state slot in place;
+    # longer chunks stage their last row and scatter it afterwards, because
+    # the chunk's first row still reads the old slot content
+    single = not getattr(md, "is_prefill", True)
     last = (torch.empty(B, W, dtype=torch.float32, device=x.device)
-            if shift is not None else None)
+            if shift is not None and not single else None)
     rc = _L().afm_dual_norm_shift(
         _lib.ptr(a), _lib.ptr(s), _lib.ptr(b), _lib.ptr(last), _lib.ptr(x),
         _lib.ptr(w1), _lib.ptr(w2), _lib.ptr(shift), _lib.ptr(prev),
@@ -132,7 +136,7 @@ def dual_norm_shift(x: torch.Tensor, w1: torch.Tensor,
         _lib.ptr(md.state_slots), float(eps), T, W, _code(a),
         _lib.cur_stream())
     _lib.check(rc, "afm_dual_norm_shift")
-    if shift is not None:
+    if last is not None:
         rc = _L().afm_scatter_state(
             _lib.ptr(prev), _lib.ptr(last), _lib.ptr(md.state_slots),
             _lib.ptr(md.cu_seqlens), B, W, _lib.cur_stream())

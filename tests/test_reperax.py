@@ -82,6 +82,24 @@ def cfg_wide_heads():
             "layers": [par], "logit_softcap": 12.0, "norm": {"eps": 1e-6}}
 
 
+def cfg_odd():
+    """Nothing divisible by 4 or 8: scalar kernel paths, odd head sizes,
+    three query heads per K/V head, a loop over the whole stack."""
+    par = {"type": "parallel", "mlp": {"ff": 25, "kind": "dense"}, "mixer": {
+        "left": {"heads": 3, "kv_heads": 1, "dim": 6, "vdim": 10,
+                 "mask": {"size": 5}, "scale": 0.5},
+        "left_scale": 1.5,
+        "right": {"heads": 3, "dim": 7, "vdim": 5, "tau": 2.5, "rank": 2},
+        "right_scale": 0.6}}
+    ret = {"type": "retention", "mlp": {"ff": 19, "kind": "dense"}, "mixer": {
+        "heads": 5, "dim": 6, "vdim": 7, "decay": [0.7, 0.8, 0.9, 0.95, 0.99],
+        "rot": {"dims": 2, "base": 77.0}}}
+    return {"architecture": "Reperax", "vocab": 33, "width": 30,
+            "layers": [par, ret], "logit_softcap": 5.0,
+            "loop": {"start": 0, "stop": 2, "times": 2},
+            "norm": {"eps": 1e-4}}
+
+
 def build(cfg_json, device, dtype, seed=0, page=8, pages=64, live=4,
           paced=True, graphs=False):
     w = orc.random_weights(cfg_json, seed, dtype)
@@ -418,7 +436,7 @@ def test_feed_forward_and_gates_alone(device, dtype):
 
 # ========================================================== whole models
 MODELS = {"mixed": cfg_mixed, "degenerate": cfg_degenerate,
-          "wide": cfg_wide_heads}
+          "wide": cfg_wide_heads, "odd": cfg_odd}
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -459,7 +477,7 @@ def test_prefill_vs_token_by_token_and_long_decode(device, dtype):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("name", ["mixed", "degenerate"])
+@pytest.mark.parametrize("name", ["mixed", "degenerate", "odd"])
 def test_portions_of_many_sizes(device, dtype, name):
     """Cuts in the middle of pages (8) and chunks (8 / 4), portions down to
     two tokens, then single tokens."""
