@@ -586,8 +586,12 @@ def _bench_config(name, width, ff, n_par, n_ret, heads, kv_heads, dim,
 
 
 HYBRID_CONFIGS = {
-    # same width / ff / depth as the Llama "tiny" and "debug-1b" configs
-    "reperax-tiny": _bench_config("reperax-tiny", 256, 512, 1, 1, 4, 2, 32,
-                                  vocab=512, chunk=32, loop=(0, 2, 2)),
+    # a small looped model for smoke runs and CPU tests
+    "reperax-tiny": _bench_config("reperax-tiny", 128, 384, 1, 1, 4, 2, 32,
+                                  vocab=384, chunk=32, loop=(0, 2, 2)),
+    # same width / ff / depth / heads as the Llama "debug-1b" config
     "reperax-1b": _bench_config("reperax-1b", 2048, 8192, 8, 8, 16, 8, 128),
+    # same width / ff / depth / heads / vocabulary as "llama-3-8b"
+    "reperax-8b": _bench_config("reperax-8b", 4096, 14336, 16, 16, 32, 8, 128,
+                                vocab=128256, chunk=1024),
 }
