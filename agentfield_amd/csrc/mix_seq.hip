@@ -188,6 +188,177 @@ __global__ void __launch_bounds__(256) masked_attention_kernel(
   }
 }
 
+// ------------------------------------------------ row attention (decode)
+// One workgroup per (row, K/V head): the GQ query heads of the group share
+// every K and V load.  Keys are walked in super-tiles of `kt`:
+//   A. scores: a key's row is read by LPK adjacent lanes, 16 bytes each
+//      (coalesced), partial dots are summed with xor-shuffles, one score per
+//      (head, key) lands in LDS; the 4 waves interleave keys;
+//   B. per head: max, exp, sum over the tile (running max / sum / rescale
+//      factor kept in LDS across super-tiles);
+//   C. P.V: a value row is read by LPV adjacent lanes, each lane accumulates
+//      its 16-byte slice for every head in registers.
+// The partial outputs of the key groups are summed with shuffles, across
+// waves through LDS.  Serves decode steps and short prompt portions, bf16
+// and fp32 storage; head sizes up to 64 lanes x 16 bytes.
+template <typename S, bool VEC>
+__device__ __forceinline__ void load_slice(const S* row, int e0, int n,
+                                           float (&o)[16 / sizeof(S)]) {
+  constexpr int EPL = 16 / sizeof(S);
+  if (VEC) {
+    if (e0 < n) {
+      if constexpr (sizeof(S) == 2) {
+        const s16x8 v = *reinterpret_cast<const s16x8*>(row + e0);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = bf2f((u16)v[j]);
+      } else {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(row + e0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = v[j];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < EPL; ++j) o[j] = 0.f;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) o[j] = (e0 + j < n) ? ldf<S>(row + e0 + j) : 0.f;
+  }
+}
+
+template <typename S, int GQ, bool VEC>
+__global__ void __launch_bounds__(256) attn_rows_kernel(
+    S* __restrict__ out, const S* __restrict__ q, const S* __restrict__ kc,
+    const S* __restrict__ vc, const i32* __restrict__ bt,
+    const i32* __restrict__ row_seq, const i32* __restrict__ positions,
+    float scale, int H, int G, int dk, int dv, int page, int maxp, int chunk,
+    int window, i64 ldq, int lpk_log2, int lpv_log2, int kt) {
+  constexpr int EPL = 16 / sizeof(S);
+  extern __shared__ float smem[];
+  const int dvp = EPL << lpv_log2;             // padded value width
+  float* sc = smem;                            // [GQ][kt] scores, then probabilities
+  float* red = sc + GQ * kt;                   // [4][GQ][dvp]
+  float* m_run = red + 4 * GQ * dvp;           // [GQ]
+  float* l_run = m_run + GQ;                   // [GQ]
+  float* corr = l_run + GQ;                    // [GQ]
+  const int t = blockIdx.x, g = blockIdx.y;
+  const int hpg = H / G;
+  const int h0 = g * hpg + blockIdx.z * GQ;
+  const int nh = min(GQ, hpg - (int)blockIdx.z * GQ);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int pos = positions[t];
+  const i32* btr = bt + (size_t)row_seq[t] * maxp;
+  int lo = 0;
+  if (chunk > 0) lo = (pos / chunk) * chunk;
+  if (window > 0 && pos - window + 1 > lo) lo = pos - window + 1;
+
+  const int lik = lane & ((1 << lpk_log2) - 1), kik = lane >> lpk_log2;
+  const int kpi = 64 >> lpk_log2;              // keys per wave iteration
+  const int liv = lane & ((1 << lpv_log2) - 1), kiv = lane >> lpv_log2;
+  const int kpv = 64 >> lpv_log2;
+
+  float qreg[GQ][EPL];
+#pragma unroll
+  for (int gg = 0; gg < GQ; ++gg)
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+      const int d = lik * EPL + j;
+      qreg[gg][j] = (gg < nh && d < dk)
+          ? ldf<S>(q + (size_t)t * ldq + (size_t)(h0 + gg) * dk + d) * scale : 0.f;
+    }
+  float acc[GQ][EPL];
+#pragma unroll
+  for (int gg = 0; gg < GQ; ++gg)
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) acc[gg][j] = 0.f;
+  if (threadIdx.x < GQ) { m_run[threadIdx.x] = AF_NEG_INF; l_run[threadIdx.x] = 0.f; }
+
+  for (int tile0 = lo; tile0 <= pos; tile0 += kt) {
+    const int nk = min(kt, pos + 1 - tile0);
+    // ---- A: scores ----
+    for (int kb = wave * kpi; kb < nk; kb += 4 * kpi) {
+      const int kidx = kb + kik;
+      const int j = tile0 + min(kidx, nk - 1);
+      const S* kr = kc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * dk;
+      float kv[EPL];
+      load_slice<S, VEC>(kr, lik * EPL, dk, kv);
+#pragma unroll
+      for (int gg = 0; gg < GQ; ++gg) {
+        float s = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) s += qreg[gg][e] * kv[e];
+        for (int o = 1; o < (1 << lpk_log2); o <<= 1) s += __shfl_xor(s, o, 64);
+        if (lik == 0 && kidx < nk && gg < nh) sc[gg * kt + kidx] = s;
+      }
+    }
+    __syncthreads();
+    // ---- B: softmax statistics, wave w takes heads w, w+4, ... ----
+    for (int gg = wave; gg < nh; gg += 4) {
+      float* sr = sc + gg * kt;
+      float mx = AF_NEG_INF;
+      for (int i = lane; i < nk; i += 64) mx = fmaxf(mx, sr[i]);
+      mx = wave_max_f32(mx);
+      const float m_old = m_run[gg];
+      const float m_new = fmaxf(m_old, mx);
+      float sum = 0.f;
+      for (int i = lane; i < nk; i += 64) {
+        const float p = expf(sr[i] - m_new);
+        sr[i] = p;
+        sum += p;
+      }
+      sum = wave_sum_f32(sum);
+      if (lane == 0) {
+        const float c = (m_old <= AF_NEG_INF) ? 0.f : expf(m_old - m_new);
+        corr[gg] = c;
+        l_run[gg] = l_run[gg] * c + sum;
+        m_run[gg] = m_new;
+      }
+    }
+    __syncthreads();
+    // ---- C: accumulate P.V ----
+    if (tile0 > lo) {
+#pragma unroll
+      for (int gg = 0; gg < GQ; ++gg) {
+        const float c = gg < nh ? corr[gg] : 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) acc[gg][e] *= c;
+      }
+    }
+    for (int kb = wave * kpv; kb < nk; kb += 4 * kpv) {
+      const int kidx = kb + kiv;
+      const bool valid = kidx < nk;
+      const int j = tile0 + min(kidx, nk - 1);
+      const S* vr = vc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * dv;
+      float vv[EPL];
+      load_slice<S, VEC>(vr, liv * EPL, dv, vv);
+#pragma unroll
+      for (int gg = 0; gg < GQ; ++gg) {
+        const float p = (valid && gg < nh) ? sc[gg * kt + kidx] : 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) acc[gg][e] += p * vv[e];
+      }
+    }
+    __syncthreads();   // scores of this tile are dead; next tile may overwrite
+  }
+  // ---- sum the key groups of a wave, then the 4 waves ----
+#pragma unroll
+  for (int gg = 0; gg < GQ; ++gg)
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      float a = acc[gg][e];
+      for (int o = 1 << lpv_log2; o < 64; o <<= 1) a += __shfl_xor(a, o, 64);
+      if (kiv == 0) red[(wave * GQ + gg) * dvp + liv * EPL + e] = a;
+    }
+  __syncthreads();
+  for (int i = threadIdx.x; i < nh * dv; i += 256) {
+    const int gg = i / dv, d = i % dv;
+    float o = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) o += red[(w * GQ + gg) * dvp + d];
+    stf<S>(out + ((size_t)t * H + h0 + gg) * dv + d, o / l_run[gg]);
+  }
+}
+
 // ------------------------------------------------------------- linear scan
 // Workgroup = (sequence, head, 32-column tile of dv); 256 threads = 16 row
 // groups x 16 column pairs.  Thread (r, c) keeps RP consecutive rows
@@ -423,6 +594,34 @@ static int launch_attention(void* out, const void* q, const void* kc,
                             const void* positions, float scale, int T, int H,
                             int G, int dk, int dv, int page, int maxp,
                             int chunk, int window, i64 ldq, hipStream_t s) {
+  constexpr int EPL = 16 / (int)sizeof(S);
+  if (dk <= 64 * EPL && dv <= 64 * EPL) {
+    auto clog2 = [](int n) { int l = 0; while ((1 << l) < n) ++l; return l; };
+    const int lpk = clog2((dk + EPL - 1) / EPL), lpv = clog2((dv + EPL - 1) / EPL);
+    const int hpg = H / G;
+    const int gq = hpg >= 8 ? 8 : hpg > 2 ? 4 : hpg;   // 1, 2, 4 or 8
+    const int dvp = EPL << lpv;
+    const int kt = dvp <= 128 ? 1024 : 512;
+    const size_t sm = ((size_t)gq * kt + 4 * gq * dvp + 3 * gq) * sizeof(float);
+    const bool vec = dk % EPL == 0 && dv % EPL == 0 &&
+                     (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0;
+    dim3 grid(T, G, (hpg + gq - 1) / gq);
+#define ROWS(GQ, VEC)                                                         \
+  attn_rows_kernel<S, GQ, VEC><<<grid, 256, sm, s>>>(                         \
+      (S*)out, (const S*)q, (const S*)kc, (const S*)vc, (const i32*)bt,       \
+      (const i32*)row_seq, (const i32*)positions, scale, H, G, dk, dv, page,  \
+      maxp, chunk, window, ldq, lpk, lpv, kt)
+    if (vec) {
+      if (gq == 1) ROWS(1, true); else if (gq == 2) ROWS(2, true);
+      else if (gq == 4) ROWS(4, true); else ROWS(8, true);
+    } else {
+      if (gq == 1) ROWS(1, false); else if (gq == 2) ROWS(2, false);
+      else if (gq == 4) ROWS(4, false); else ROWS(8, false);
+    }
+#undef ROWS
+    return af_last_err();
+  }
+  // very wide heads: one wave per (row, head), scalar key walk
   const int n_rh = T * H;
   const int grid = (n_rh + 3) / 4;
   const size_t sm = (size_t)4 * (dk + 64) * sizeof(float);

@@ -379,13 +379,17 @@ class ReperaxLayer(nn.Module):
         # one GEMM feeds every projection that reads the shifted input
         self.blocks = [(mn, bn, rows) for mn, m in self.mixers.items()
                        for bn, rows in m.in_blocks()]
+        # fused weights are padded to 64 output rows (the skinny decode GEMM's
+        # tile); the padding rows produce columns nobody reads
+        def pad64(n):
+            return n + (-n) % 64
         self.mix_in = nn.Parameter(torch.empty(
-            sum(r for _, _, r in self.blocks), W))
+            pad64(sum(r for _, _, r in self.blocks)), W))
         if spec.ff is not None:
             self.norm2 = nn.Parameter(torch.empty(W))
             self.mlp = PolyNormMLP(spec.ff, W, eps)
             # [up | output-gate logits]: both read norm2(x)
-            self.ff_in = nn.Parameter(torch.empty(spec.ff + W, W))
+            self.ff_in = nn.Parameter(torch.empty(pad64(spec.ff + W), W))
             self.register_buffer("rg2_b", torch.zeros(W, dtype=torch.float32))
         else:
             self.norm2 = None
@@ -407,7 +411,8 @@ class ReperaxLayer(nn.Module):
         if self.mlp is not None:
             u = sm.matmul(b, self.ff_in)
             m_out = self.mlp(u[:, :self.spec.ff])
-            g2, b2 = u[:, self.spec.ff:], self.rg2_b
+            g2 = u[:, self.spec.ff:self.spec.ff + x.shape[1]]
+            b2 = self.rg2_b
         sm.gated_residual(x, outs[0], self.scales[0],
                           outs[1] if len(outs) > 1 else None,
                           self.scales[1] if len(outs) > 1 else 0.0,
@@ -463,7 +468,9 @@ class ReperaxForCausalLM(nn.Module):
                 self.record_runs.append(x.clone())
         h = sm.norm_rows(x, self.final_norm, cfg.eps, logit_rows,
                          self.embed.dtype)
-        return sm.softcap(sm.matmul(h, self.embed), cfg.logit_softcap)
+        # vocabulary-sized N: the vendor GEMM wins there at every row count
+        return sm.softcap(sm.matmul(h, self.embed, skinny=False),
+                          cfg.logit_softcap)
 
     # -- weights ------------------------------------------------------------
     @torch.no_grad()
@@ -485,8 +492,14 @@ class ReperaxForCausalLM(nn.Module):
             put(L.rg1, get(pre + "rg1"))
             put(L.rg1_b, get(pre + "rg1.b"))
             sub = {"left": "mix.left.", "right": "mix.right.", "ret": "mix."}
+            def padded(parts, total):
+                t = torch.cat(parts, 0)
+                if t.shape[0] < total:
+                    t = torch.cat([t, t.new_zeros(total - t.shape[0],
+                                                  t.shape[1])], 0)
+                return t
             rows = [get(pre + sub[mn] + bn) for mn, bn, _ in L.blocks]
-            put(L.mix_in, torch.cat(rows, 0))
+            put(L.mix_in, padded(rows, L.mix_in.shape[0]))
             for mn, m in L.mixers.items():
                 mp = pre + sub[mn]
                 put(m.o, get(mp + "o"))
@@ -499,8 +512,8 @@ class ReperaxForCausalLM(nn.Module):
                     put(m.norm, get(mp + "norm"))
             if L.mlp is not None:
                 put(L.norm2, get(pre + "norm2"))
-                put(L.ff_in, torch.cat([get(pre + "mlp.up"),
-                                        get(pre + "rg2")], 0))
+                put(L.ff_in, padded([get(pre + "mlp.up"), get(pre + "rg2")],
+                                    L.ff_in.shape[0]))
                 put(L.rg2_b, get(pre + "rg2.b"))
                 put(L.mlp.down, get(pre + "mlp.down"))
                 put(L.mlp.act, get(pre + "mlp.act"))

@@ -146,6 +146,11 @@ def check(rc: int, name: str) -> None:
         raise AfOpsError(f"{name} failed with code {rc} (hipError or 9xxx arg check)")
 
 
+def main_lib_ready() -> bool:
+    """True when libafops.so is on disk (never triggers a build)."""
+    return _LIB_PATH.exists()
+
+
 def native_loaded() -> bool:
     try:
         lib()

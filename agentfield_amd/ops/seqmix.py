@@ -428,7 +428,22 @@ def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
     return out
 
 
-def matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """x [M, K] @ w [N, K]^T through the vendor GEMM (hipBLASLt / rocBLAS);
-    fp32 operands run in true fp32 (no reduced-precision matrix mode)."""
+def matmul(x: torch.Tensor, w: torch.Tensor,
+           skinny: bool = True) -> torch.Tensor:
+    """x [M, K] @ w [N, K]^T.  Decode-sized bf16 products (few rows, weight
+    streaming bound) go to the framework's MFMA skinny-GEMM kernel when its
+    library is built and the shape fits it (N, K multiples of 64) — the same
+    per-shape policy ops.linear measured for the Llama family; everything
+    else is the vendor GEMM (hipBLASLt / rocBLAS), fp32 operands in true
+    fp32 (no reduced-precision matrix mode)."""
+    M, K = x.shape
+    N = w.shape[0]
+    if (skinny and x.is_cuda and x.dtype == torch.bfloat16
+            and N % 64 == 0 and K % 64 == 0
+            and ((M <= 64 and K <= 8192)
+                 or (32 < M <= 128 and K >= 8192 and N <= 8192))
+            and x.is_contiguous() and w.is_contiguous()
+            and _lib.main_lib_ready()):
+        from . import linear_skinny
+        return linear_skinny(x, w)
     return x @ w.t()
