@@ -191,9 +191,9 @@ __global__ void __launch_bounds__(256) masked_attention_kernel(
 // ------------------------------------------------ row attention (decode)
 // One workgroup per (row, K/V head): the GQ query heads of the group share
 // every K and V load.  Keys are walked in super-tiles of `kt`:
-//   A. scores: a key's row is read by LPK adjacent lanes, 16 bytes each
-//      (coalesced), partial dots are summed with xor-shuffles, one score per
-//      (head, key) lands in LDS; the 4 waves interleave keys;
+//   A. scores: one key per lane, its row read 16 bytes at a time and dotted
+//      with every head's query (queries sit in LDS, read as broadcasts), so
+//      no cross-lane reduction is needed; one score per (head, key) in LDS;
 //   B. per head: max, exp, sum over the tile (running max / sum / rescale
 //      factor kept in LDS across super-tiles);
 //   C. P.V: a value row is read by LPV adjacent lanes, each lane accumulates
@@ -232,40 +232,47 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
     const S* __restrict__ vc, const i32* __restrict__ bt,
     const i32* __restrict__ row_seq, const i32* __restrict__ positions,
     float scale, int H, int G, int dk, int dv, int page, int maxp, int chunk,
-    int window, i64 ldq, int lpk_log2, int lpv_log2, int kt) {
+    int window, i64 ldq, int lpk_log2, int lpv_log2, int kt, int nsplit,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
+  // nsplit > 1: the visible keys are cut into nsplit ranges, one workgroup
+  // each (grid.z = head blocks x nsplit); unnormalised outputs and (max,
+  // sum) go to part_o [T, H, nsplit, dv] / part_ml [T, H, nsplit, 2] and
+  // attn_split_combine_kernel merges them.
   constexpr int EPL = 16 / sizeof(S);
   extern __shared__ float smem[];
   const int dvp = EPL << lpv_log2;             // padded value width
   float* sc = smem;                            // [GQ][kt] scores, then probabilities
   float* red = sc + GQ * kt;                   // [4][GQ][dvp]
-  float* m_run = red + 4 * GQ * dvp;           // [GQ]
-  float* l_run = m_run + GQ;                   // [GQ]
-  float* corr = l_run + GQ;                    // [GQ]
+  float* m_run = red + 4 * GQ * dvp;           // [8]
+  float* l_run = m_run + 8;                    // [8]
+  float* corr = l_run + 8;                     // [8]
+  const int dkp = (dk + EPL - 1) / EPL * EPL;
+  float* qs = corr + 8;                        // [GQ][dkp] scaled queries
   const int t = blockIdx.x, g = blockIdx.y;
   const int hpg = H / G;
-  const int h0 = g * hpg + blockIdx.z * GQ;
-  const int nh = min(GQ, hpg - (int)blockIdx.z * GQ);
+  const int zh = blockIdx.z / nsplit, sp = blockIdx.z % nsplit;
+  const int h0 = g * hpg + zh * GQ;
+  const int nh = min(GQ, hpg - zh * GQ);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int pos = positions[t];
+  int pos = positions[t];
   const i32* btr = bt + (size_t)row_seq[t] * maxp;
   int lo = 0;
   if (chunk > 0) lo = (pos / chunk) * chunk;
   if (window > 0 && pos - window + 1 > lo) lo = pos - window + 1;
+  if (nsplit > 1) {   // this workgroup's share of [lo, pos]; may be empty
+    const int per = (pos - lo + nsplit) / nsplit;
+    lo += sp * per;
+    pos = min(pos, lo + per - 1);
+  }
 
-  const int lik = lane & ((1 << lpk_log2) - 1), kik = lane >> lpk_log2;
-  const int kpi = 64 >> lpk_log2;              // keys per wave iteration
   const int liv = lane & ((1 << lpv_log2) - 1), kiv = lane >> lpv_log2;
   const int kpv = 64 >> lpv_log2;
 
-  float qreg[GQ][EPL];
-#pragma unroll
-  for (int gg = 0; gg < GQ; ++gg)
-#pragma unroll
-    for (int j = 0; j < EPL; ++j) {
-      const int d = lik * EPL + j;
-      qreg[gg][j] = (gg < nh && d < dk)
-          ? ldf<S>(q + (size_t)t * ldq + (size_t)(h0 + gg) * dk + d) * scale : 0.f;
-    }
+  for (int i = threadIdx.x; i < GQ * dkp; i += 256) {
+    const int gg = i / dkp, d = i % dkp;
+    qs[i] = (gg < nh && d < dk)
+        ? ldf<S>(q + (size_t)t * ldq + (size_t)(h0 + gg) * dk + d) * scale : 0.f;
+  }
   float acc[GQ][EPL];
 #pragma unroll
   for (int gg = 0; gg < GQ; ++gg)
@@ -275,21 +282,26 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
 
   for (int tile0 = lo; tile0 <= pos; tile0 += kt) {
     const int nk = min(kt, pos + 1 - tile0);
-    // ---- A: scores ----
-    for (int kb = wave * kpi; kb < nk; kb += 4 * kpi) {
-      const int kidx = kb + kik;
-      const int j = tile0 + min(kidx, nk - 1);
+    // ---- A: scores, one key per lane ----
+    if (tile0 == lo) __syncthreads();          // queries are in LDS
+    for (int kidx = threadIdx.x; kidx < nk; kidx += 256) {
+      const int j = tile0 + kidx;
       const S* kr = kc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * dk;
-      float kv[EPL];
-      load_slice<S, VEC>(kr, lik * EPL, dk, kv);
+      float sco[GQ];
 #pragma unroll
-      for (int gg = 0; gg < GQ; ++gg) {
-        float s = 0.f;
+      for (int gg = 0; gg < GQ; ++gg) sco[gg] = 0.f;
+#pragma unroll 4
+      for (int e0 = 0; e0 < dk; e0 += EPL) {
+        float kv[EPL];
+        load_slice<S, VEC>(kr, e0, dk, kv);
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) s += qreg[gg][e] * kv[e];
-        for (int o = 1; o < (1 << lpk_log2); o <<= 1) s += __shfl_xor(s, o, 64);
-        if (lik == 0 && kidx < nk && gg < nh) sc[gg * kt + kidx] = s;
+        for (int gg = 0; gg < GQ; ++gg)
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) sco[gg] += qs[gg * dkp + e0 + e] * kv[e];
       }
+#pragma unroll
+      for (int gg = 0; gg < GQ; ++gg)
+        if (gg < nh) sc[gg * kt + kidx] = sco[gg];
     }
     __syncthreads();
     // ---- B: softmax statistics, wave w takes heads w, w+4, ... ----
@@ -324,18 +336,24 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
         for (int e = 0; e < EPL; ++e) acc[gg][e] *= c;
       }
     }
-    for (int kb = wave * kpv; kb < nk; kb += 4 * kpv) {
-      const int kidx = kb + kiv;
-      const bool valid = kidx < nk;
-      const int j = tile0 + min(kidx, nk - 1);
-      const S* vr = vc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * dv;
-      float vv[EPL];
-      load_slice<S, VEC>(vr, liv * EPL, dv, vv);
+    for (int kb = wave * kpv; kb < nk; kb += 16 * kpv) {
+      float vv[4][EPL];
 #pragma unroll
-      for (int gg = 0; gg < GQ; ++gg) {
-        const float p = (valid && gg < nh) ? sc[gg * kt + kidx] : 0.f;
+      for (int u = 0; u < 4; ++u) {
+        const int j = tile0 + min(kb + u * 4 * kpv + kiv, nk - 1);
+        const S* vr = vc + (((size_t)btr[j / page] * G + g) * page + (j % page)) * dv;
+        load_slice<S, VEC>(vr, liv * EPL, dv, vv[u]);
+      }
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) acc[gg][e] += p * vv[e];
+      for (int u = 0; u < 4; ++u) {
+        const int kidx = kb + u * 4 * kpv + kiv;
+        const bool valid = kidx < nk;
+#pragma unroll
+        for (int gg = 0; gg < GQ; ++gg) {
+          const float p = (valid && gg < nh) ? sc[gg * kt + kidx] : 0.f;
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) acc[gg][e] += p * vv[u][e];
+        }
       }
     }
     __syncthreads();   // scores of this tile are dead; next tile may overwrite
@@ -355,7 +373,38 @@ __global__ void __launch_bounds__(256) attn_rows_kernel(
     float o = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) o += red[(w * GQ + gg) * dvp + d];
-    stf<S>(out + ((size_t)t * H + h0 + gg) * dv + d, o / l_run[gg]);
+    if (nsplit == 1)
+      stf<S>(out + ((size_t)t * H + h0 + gg) * dv + d, o / l_run[gg]);
+    else
+      part_o[(((size_t)t * H + h0 + gg) * nsplit + sp) * dv + d] = o;
+  }
+  if (nsplit > 1 && threadIdx.x < nh) {
+    float* ml = part_ml + (((size_t)t * H + h0 + threadIdx.x) * nsplit + sp) * 2;
+    ml[0] = m_run[threadIdx.x];
+    ml[1] = l_run[threadIdx.x];
+  }
+}
+
+// One wave per (row, head): merge the nsplit partial softmaxes.
+template <typename S>
+__global__ void __launch_bounds__(256) attn_split_combine_kernel(
+    S* __restrict__ out, const float* __restrict__ part_o,
+    const float* __restrict__ part_ml, int n_rh, int nsplit, int dv) {
+  const int rh = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (rh >= n_rh) return;
+  const int lane = threadIdx.x & 63;
+  const float* ml = part_ml + (size_t)rh * nsplit * 2;
+  float m = AF_NEG_INF;
+  for (int s = 0; s < nsplit; ++s) m = fmaxf(m, ml[2 * s]);
+  float l = 0.f;
+  for (int s = 0; s < nsplit; ++s)
+    if (ml[2 * s] > AF_NEG_INF) l += ml[2 * s + 1] * expf(ml[2 * s] - m);
+  for (int d = lane; d < dv; d += 64) {
+    float o = 0.f;
+    for (int s = 0; s < nsplit; ++s)
+      if (ml[2 * s] > AF_NEG_INF)
+        o += part_o[((size_t)rh * nsplit + s) * dv + d] * expf(ml[2 * s] - m);
+    stf<S>(out + (size_t)rh * dv + d, o / l);
   }
 }
 
@@ -593,7 +642,8 @@ static int launch_attention(void* out, const void* q, const void* kc,
                             const void* vc, const void* bt, const void* row_seq,
                             const void* positions, float scale, int T, int H,
                             int G, int dk, int dv, int page, int maxp,
-                            int chunk, int window, i64 ldq, hipStream_t s) {
+                            int chunk, int window, i64 ldq, int nsplit,
+                            float* part_o, float* part_ml, hipStream_t s) {
   constexpr int EPL = 16 / (int)sizeof(S);
   if (dk <= 64 * EPL && dv <= 64 * EPL) {
     auto clog2 = [](int n) { int l = 0; while ((1 << l) < n) ++l; return l; };
@@ -602,15 +652,18 @@ static int launch_attention(void* out, const void* q, const void* kc,
     const int gq = hpg >= 8 ? 8 : hpg > 2 ? 4 : hpg;   // 1, 2, 4 or 8
     const int dvp = EPL << lpv;
     const int kt = dvp <= 128 ? 1024 : 512;
-    const size_t sm = ((size_t)gq * kt + 4 * gq * dvp + 3 * gq) * sizeof(float);
+    const int dkp = (dk + EPL - 1) / EPL * EPL;
+    const size_t sm = ((size_t)gq * kt + 4 * gq * dvp + 24 +
+                       (size_t)gq * dkp) * sizeof(float);
     const bool vec = dk % EPL == 0 && dv % EPL == 0 &&
                      (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0;
-    dim3 grid(T, G, (hpg + gq - 1) / gq);
+    if (nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) return 9003;
+    dim3 grid(T, G, ((hpg + gq - 1) / gq) * nsplit);
 #define ROWS(GQ, VEC)                                                         \
   attn_rows_kernel<S, GQ, VEC><<<grid, 256, sm, s>>>(                         \
       (S*)out, (const S*)q, (const S*)kc, (const S*)vc, (const i32*)bt,       \
       (const i32*)row_seq, (const i32*)positions, scale, H, G, dk, dv, page,  \
-      maxp, chunk, window, ldq, lpk, lpv, kt)
+      maxp, chunk, window, ldq, lpk, lpv, kt, nsplit, part_o, part_ml)
     if (vec) {
       if (gq == 1) ROWS(1, true); else if (gq == 2) ROWS(2, true);
       else if (gq == 4) ROWS(4, true); else ROWS(8, true);
@@ -619,6 +672,9 @@ static int launch_attention(void* out, const void* q, const void* kc,
       else if (gq == 4) ROWS(4, false); else ROWS(8, false);
     }
 #undef ROWS
+    if (nsplit > 1)
+      attn_split_combine_kernel<S><<<(T * H + 3) / 4, 256, 0, s>>>(
+          (S*)out, part_o, part_ml, T * H, nsplit, dv);
     return af_last_err();
   }
   // very wide heads: one wave per (row, head), scalar key walk
@@ -641,18 +697,20 @@ AF_EXPORT int afm_masked_attention(
     void* out, const void* q, const void* kc, const void* vc, const void* bt,
     const void* row_seq, const void* positions, float scale, int T, int H,
     int G, int dk, int dv, int page, int maxp, int chunk, int window, i64 ldq,
-    int dt, void* stream) {
+    int nsplit, void* part_o, void* part_ml, int dt, void* stream) {
   if (T == 0) return 0;
   if (G <= 0 || H % G || dv > 256 || dk > 1024) return 9003;
   hipStream_t s = (hipStream_t)stream;
   if (dt == 0)
     return launch_attention<u16>(out, q, kc, vc, bt, row_seq, positions, scale,
                                  T, H, G, dk, dv, page, maxp, chunk, window,
-                                 ldq, s);
+                                 ldq, nsplit, (float*)part_o, (float*)part_ml,
+                                 s);
   if (dt == 1)
     return launch_attention<float>(out, q, kc, vc, bt, row_seq, positions,
                                    scale, T, H, G, dk, dv, page, maxp, chunk,
-                                   window, ldq, s);
+                                   window, ldq, nsplit, (float*)part_o,
+                                   (float*)part_ml, s);
   return 9002;
 }
 

@@ -119,7 +119,7 @@ def _declare_mix(l: ctypes.CDLL) -> None:
         "afm_qk_norm_cache": [p, p, p, p, p, p, p, p, p, f, i, i, i, i, i, i,
                               i, i, i64, i64, i64, i, p],
         "afm_masked_attention": [p, p, p, p, p, p, p, f, i, i, i, i, i, i, i,
-                                 i, i, i64, i, p],
+                                 i, i, i64, i, p, p, i, p],
         "afm_attn_prefill_mfma": [p, p, p, p, p, p, p, p, p, f, i, i, i, i, i,
                                   i, i, i, i, i64, p],
         "afm_linear_scan": [p, p, p, p, p, p, p, p, p, p, p, p, p, f, f, f,

@@ -255,11 +255,25 @@ def masked_attention(q: torch.Tensor, kcache: torch.Tensor,
             _lib.cur_stream())
         _lib.check(rc, "afm_attn_prefill_mfma")
         return out
+    # few rows and many visible keys: cut the keys over several workgroups
+    # (about 2048 in flight) and merge the partial softmaxes
+    reach = min(x for x in (chunk, window, md.block_table.shape[1] * page)
+                if x > 0)
+    per_wg_heads = min(8, max(1, H // G))
+    wgs = T * G * -(-(H // G) // per_wg_heads)
+    nsplit = max(1, min(8, 2048 // max(1, wgs), reach // 128))
+    part_o = part_ml = None
+    if nsplit > 1:
+        part_o = torch.empty(T, H, nsplit, dv, dtype=torch.float32,
+                             device=q.device)
+        part_ml = torch.empty(T, H, nsplit, 2, dtype=torch.float32,
+                              device=q.device)
     rc = _L().afm_masked_attention(
         _lib.ptr(out), _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vcache),
         _lib.ptr(md.block_table), _lib.ptr(md.row_seq), _lib.ptr(positions),
         float(scale), T, H, G, dk, dv, page, md.block_table.shape[1],
-        int(chunk), int(window), _rowstride(q), _code(q), _lib.cur_stream())
+        int(chunk), int(window), _rowstride(q), nsplit, _lib.ptr(part_o),
+        _lib.ptr(part_ml), _code(q), _lib.cur_stream())
     _lib.check(rc, "afm_masked_attention")
     return out
 
