@@ -20,6 +20,7 @@ do not depend on where a prompt was cut into chunks.
 from __future__ import annotations
 
 import math
+import os
 
 import torch
 
@@ -29,6 +30,7 @@ _DT = {torch.bfloat16: 0, torch.float32: 1}
 # a step whose longest row chunk reaches this many rows runs bf16 attention
 # through the MFMA tile kernel; shorter steps (decode) use one wave per row
 MFMA_MIN_ROWS = 16
+_SKINNY = os.environ.get("AF_MIX_SKINNY", "0") == "1"
 
 
 def _gpu(t: torch.Tensor) -> bool:
@@ -444,15 +446,19 @@ def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
 
 def matmul(x: torch.Tensor, w: torch.Tensor,
            skinny: bool = True) -> torch.Tensor:
-    """x [M, K] @ w [N, K]^T.  Decode-sized bf16 products (few rows, weight
-    streaming bound) go to the framework's MFMA skinny-GEMM kernel when its
-    library is built and the shape fits it (N, K multiples of 64) — the same
-    per-shape policy ops.linear measured for the Llama family; everything
-    else is the vendor GEMM (hipBLASLt / rocBLAS), fp32 operands in true
-    fp32 (no reduced-precision matrix mode)."""
+    """x [M, K] @ w [N, K]^T through the vendor GEMM (hipBLASLt / rocBLAS);
+    fp32 operands run in true fp32 (no reduced-precision matrix mode).
+
+    AF_MIX_SKINNY=1 sends decode-sized bf16 products (<= 64 rows, N and K
+    multiples of 64) to the framework's MFMA skinny-GEMM kernel instead, with
+    the per-shape policy ops.linear uses for the Llama family.  Measured on
+    MI355X for this family the two are equal in GEMM time (1.33 vs 1.34 ms
+    per 64-row step at width 2048, and the same tokens/s at width 4096) while
+    the skinny path adds a combine launch per product, so the vendor GEMM is
+    the default."""
     M, K = x.shape
     N = w.shape[0]
-    if (skinny and x.is_cuda and x.dtype == torch.bfloat16
+    if (skinny and _SKINNY and x.is_cuda and x.dtype == torch.bfloat16
             and N % 64 == 0 and K % 64 == 0
             and ((M <= 64 and K <= 8192)
                  or (32 < M <= 128 and K >= 8192 and N <= 8192))
