@@ -219,7 +219,8 @@ def test_dual_norm_shift_and_state(device, dtype):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(3, 1, 8, 8, 4), (4, 2, 12, 20, 8),
-                                   (2, 1, 72, 80, 96), (6, 6, 16, 16, 0)])
+                                   (2, 1, 72, 80, 96), (6, 6, 16, 16, 0),
+                                   (2, 1, 264, 24, 16), (10, 1, 16, 8, 32)])
 def test_chunk_attention_alone(device, dtype, shape):
     H, G, dk, dv, chunk = shape
     torch.manual_seed(2)
