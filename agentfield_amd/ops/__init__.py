@@ -452,3 +452,9 @@ def mfma_probe(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
                                   _lib.cur_stream())
     _lib.check(rc, "af_mfma_probe")
     return d
+
+
+# the sequence-mixer op set (masked attention for any head size, decayed
+# recurrences with state slots, hybrid-decoder glue) lives in its own module
+# and kernel library
+from . import seqmix  # noqa: E402,F401
