@@ -38,11 +38,20 @@ HIP_SOURCES = [
     "probe.hip",
 ]
 
-# Kernel groups that build into their own small library, so a process that
-# serves only one model family compiles (and loads) only what it runs.
-# libafmix.so: sequence-mixer op set (ops/seqmix.py).
-MIX_SOURCES = ["mix_glue.hip", "mix_seq.hip", "mix_attn_mfma.hip"]
-MIX_LIB = PKG_DIR / "libafmix.so"
+# Kernel groups that build into their own small libraries, so a process that
+# serves only one model family compiles (and loads) only what it runs
+# (ops/seqmix.py resolves each entry point to its group):
+#   glue    row-wise glue shared by the hybrid families (embedding to an fp32
+#           residual, norms, gated units, routers)
+#   seq     masked softmax attention + decayed linear recurrences
+#   ssm     selective state-space scan + sigmoid attention
+MIX_GROUPS = {
+    "glue": (PKG_DIR / "libafglue.so", ["mix_glue.hip"]),
+    "seq": (PKG_DIR / "libafmix.so", ["mix_seq.hip", "mix_attn_mfma.hip"]),
+    "ssm": (PKG_DIR / "libafssm.so", ["mix_ssm.hip", "mix_sigattn.hip"]),
+}
+MIX_SOURCES = [s for _lib, srcs in MIX_GROUPS.values() for s in srcs]
+MIX_LIB = MIX_GROUPS["seq"][0]
 
 # hipcc -O3 may otherwise fuse scalar float code into packed-fp32 VALU ops
 HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -58,9 +67,15 @@ def _needs_build(lib: Path = LIB, sources=None) -> bool:
     return any(d.stat().st_mtime > lib_m for d in deps)
 
 
-def build_mix(force: bool = False, verbose: bool = True) -> Path:
-    """Compile the sequence-mixer kernel group (libafmix.so) for gfx950."""
-    return _build_lib(MIX_LIB, MIX_SOURCES, force, verbose)
+def build_mix(force: bool = False, verbose: bool = True,
+              group: str | None = None):
+    """Compile the sequence-mixer kernel groups for gfx950 (one group, or
+    all of them); returns the library path(s)."""
+    if group is not None:
+        lib, srcs = MIX_GROUPS[group]
+        return _build_lib(lib, srcs, force, verbose)
+    return [_build_lib(lib, srcs, force, verbose)
+            for lib, srcs in MIX_GROUPS.values()]
 
 
 def build_afops(force: bool = False, verbose: bool = True) -> Path:

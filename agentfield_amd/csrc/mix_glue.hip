@@ -303,6 +303,170 @@ __global__ void __launch_bounds__(256) softcap_kernel(
   }
 }
 
+// fp32 rows -> storage dtype (the projections' input when sublayers read the
+// residual itself).
+template <typename S>
+__global__ void __launch_bounds__(256) cast_rows_kernel(
+    S* __restrict__ out, const float* __restrict__ x, i64 n) {
+  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (i64)gridDim.x * 256)
+    stf<S>(out + i, x[i]);
+}
+
+// Norm on a sublayer's OUTPUT, then the residual add:
+//   u = y (+ bias);  x += u / sqrt(mean(u^2) + eps) * w;  h = S(x)
+// y is [T, W] in Y (storage dtype or fp32), x the fp32 residual, h an
+// optional copy of the new residual row in the storage dtype.
+template <typename S, typename Y>
+__global__ void __launch_bounds__(256) norm_residual_kernel(
+    float* __restrict__ x, S* __restrict__ h, const Y* __restrict__ y,
+    i64 ldy, const S* __restrict__ bias, const S* __restrict__ w, float eps,
+    int W) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const Y* yr = y + (size_t)t * ldy;
+  float ss[1] = {0.f};
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const float u = ldf<Y>(yr + i) + (bias ? ldf<S>(bias + i) : 0.f);
+    ss[0] += u * u;
+  }
+  block_sum<1>(ss, red);
+  const float rs = 1.0f / sqrtf(ss[0] / (float)W + eps);
+  float* xr = x + (size_t)t * W;
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const float u = ldf<Y>(yr + i) + (bias ? ldf<S>(bias + i) : 0.f);
+    const float v = xr[i] + u * rs * ldf<S>(w + i);
+    xr[i] = v;
+    if (h) stf<S>(h + (size_t)t * W + i, v);
+  }
+}
+
+// Gated linear unit over rows of [gate | up]:
+//   out[r, i] = act(g[r, i] + bg[i]) * (u[r, i] + bu[i]) * rw[r]
+// act: 0 SiLU, 1 ReLU, 2 tanh-GELU.  Biases and the per-row weight rw (fp32,
+// e.g. a router weight per (token, expert) row) are optional.  Row r sits at
+// (r / rg) * ld + (r % rg) * ld_in, so rg units laid side by side in one
+// matrix row (experts of one token) are rows of their own.
+template <typename S, int ACT>
+__global__ void __launch_bounds__(256) glu_kernel(
+    S* __restrict__ out, i64 ldo, i64 ldo_in, const S* __restrict__ g,
+    const S* __restrict__ u, i64 ldi, i64 ldi_in, int rg,
+    const S* __restrict__ bg, const S* __restrict__ bu,
+    const float* __restrict__ rw, i64 R, int F) {
+  const i64 n = R * F;
+  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (i64)gridDim.x * 256) {
+    const i64 r = i / F;
+    const int c = (int)(i % F);
+    const i64 ri = (r / rg) * ldi + (r % rg) * ldi_in;
+    float a = ldf<S>(g + ri + c) + (bg ? ldf<S>(bg + c) : 0.f);
+    const float b = ldf<S>(u + ri + c) + (bu ? ldf<S>(bu + c) : 0.f);
+    if (ACT == 0) a = a / (1.0f + expf(-a));
+    else if (ACT == 1) a = fmaxf(a, 0.f);
+    else a = 0.5f * a * (1.0f + tanhf(0.7978845608028654f *
+                                      (a + 0.044715f * a * a * a)));
+    float o = a * b;
+    if (rw) o *= rw[r];
+    stf<S>(out + (r / rg) * ldo + (r % rg) * ldo_in + c, o);
+  }
+}
+
+// Sigmoid router with score correction and group-limited top-k, one wave per
+// token.  z [T, E] fp32 logits; s = sigmoid(z); choice = s + corr.  With
+// n_groups > 0 the experts form n_groups equal groups of neighbours, a
+// group's score is the sum of its two largest choice scores, and experts
+// outside the best `keep` groups cannot be chosen.  The `top` largest choice
+// scores win (ties: lower index); weights = s / (sum of chosen s + 1e-20) *
+// scale.  Outputs idx [T, top] i32, wts [T, top] fp32 and, optionally, the
+// dense form wd [T, E] fp32 (zero for experts not chosen).
+__global__ void __launch_bounds__(64) moe_route_kernel(
+    i32* __restrict__ idx, float* __restrict__ wts, float* __restrict__ wd,
+    const float* __restrict__ z, const float* __restrict__ corr, int E,
+    int top, int n_groups, int keep, float scale) {
+  extern __shared__ float sh[];
+  float* sig = sh;             // [E]
+  float* choice = sh + E;      // [E]
+  float* gsc = sh + 2 * E;     // [n_groups]
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const float* zr = z + (size_t)t * E;
+  for (int e = lane; e < E; e += 64) {
+    const float s = 1.0f / (1.0f + expf(-zr[e]));
+    sig[e] = s;
+    choice[e] = s + (corr ? corr[e] : 0.f);
+    if (wd) wd[(size_t)t * E + e] = 0.f;
+  }
+  __syncthreads();
+  if (n_groups > 0 && keep < n_groups) {
+    const int size = E / n_groups;
+    for (int g = lane; g < n_groups; g += 64) {
+      float a = -INFINITY, b = -INFINITY;   // largest, second largest
+      for (int m = 0; m < size; ++m) {
+        const float c = choice[g * size + m];
+        if (c > a) { b = a; a = c; }
+        else if (c > b) b = c;
+      }
+      gsc[g] = size > 1 ? a + b : a;
+    }
+    __syncthreads();
+    for (int g = lane; g < n_groups; g += 64) {
+      const float mine = gsc[g];
+      int rank = 0;
+      for (int o = 0; o < n_groups; ++o)
+        rank += (gsc[o] > mine || (gsc[o] == mine && o < g)) ? 1 : 0;
+      if (rank >= keep)
+        for (int m = 0; m < size; ++m) choice[g * size + m] = -INFINITY;
+    }
+    __syncthreads();
+  }
+  float total = 0.f;
+  for (int r = 0; r < top; ++r) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float c = choice[e];
+      if (c > bv) { bv = c; bi = e; }   // ascending e: first of equals stays
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if (bi >= E) bi = r < E ? r : 0;    // fewer candidates than `top`
+    total += sig[bi];
+    if (lane == 0) {
+      idx[(size_t)t * top + r] = bi;
+      wts[(size_t)t * top + r] = sig[bi];
+      choice[bi] = -INFINITY;
+    }
+    __syncthreads();
+  }
+  const float inv = scale / (total + 1e-20f);
+  for (int r = lane; r < top; r += 64) {
+    const float w = wts[(size_t)t * top + r] * inv;
+    wts[(size_t)t * top + r] = w;
+    if (wd) wd[(size_t)t * E + idx[(size_t)t * top + r]] = w;
+  }
+}
+
+// y[t] = sum_r wts[t, r] * ys[pos[t*top + r]] (+ shared[t]) in fp32, the sum
+// taken in the order r = 0 .. top-1.  ys rows sit in expert-sorted order; pos
+// is the inverse of that sort.
+template <typename S>
+__global__ void __launch_bounds__(256) moe_combine_kernel(
+    float* __restrict__ y, const S* __restrict__ ys,
+    const i32* __restrict__ pos, const float* __restrict__ wts,
+    const S* __restrict__ shared, int top, int W) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < W; i += 256) {
+    float acc = shared ? ldf<S>(shared + (size_t)t * W + i) : 0.f;
+    for (int r = 0; r < top; ++r)
+      acc += wts[(size_t)t * top + r] *
+             ldf<S>(ys + (size_t)pos[(size_t)t * top + r] * W + i);
+    y[(size_t)t * W + i] = acc;
+  }
+}
+
 template <typename... P>
 inline bool aligned16(P... p) {
   return ((((uintptr_t)p) % 16 == 0) && ...);
@@ -449,5 +613,87 @@ AF_EXPORT int afm_softcap(void* out, const void* in, float cap, i64 n, int dt,
           (const u16*)in, cap, n)),
       (softcap_kernel<float><<<grid_for(n), 256, 0, s>>>((float*)out,
           (const float*)in, cap, n)));
+  return af_last_err();
+}
+
+AF_EXPORT int afm_cast_rows(void* out, const void* x, i64 n, int dt,
+                            void* stream) {
+  if (n == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  MIX_DISPATCH(dt,
+      (cast_rows_kernel<u16><<<grid_for(n), 256, 0, s>>>((u16*)out,
+          (const float*)x, n)),
+      (cast_rows_kernel<float><<<grid_for(n), 256, 0, s>>>((float*)out,
+          (const float*)x, n)));
+  return af_last_err();
+}
+
+// y_f32 != 0: y holds fp32 whatever the storage dtype.
+AF_EXPORT int afm_norm_residual(void* x, void* h, const void* y, i64 ldy,
+                                int y_f32, const void* bias, const void* w,
+                                float eps, int T, int W, int dt,
+                                void* stream) {
+  if (T == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+#define NR(ST, YT)                                                          \
+  norm_residual_kernel<ST, YT><<<T, 256, 0, s>>>((float*)x, (ST*)h,         \
+      (const YT*)y, ldy, (const ST*)bias, (const ST*)w, eps, W)
+  if (dt == 0) { if (y_f32) NR(u16, float); else NR(u16, u16); }
+  else if (dt == 1) NR(float, float);
+  else return 9002;
+#undef NR
+  return af_last_err();
+}
+
+AF_EXPORT int afm_glu(void* out, i64 ldo, i64 ldo_in, const void* g,
+                      const void* u, i64 ldi, i64 ldi_in, int rg,
+                      const void* bg, const void* bu, const void* rw, i64 R,
+                      int F, int act, int dt, void* stream) {
+  if (R == 0 || F == 0) return 0;
+  if (act < 0 || act > 2 || rg < 1) return 9003;
+  hipStream_t s = (hipStream_t)stream;
+  const int grid = grid_for(R * F);
+#define GLU(ST, A)                                                         \
+  glu_kernel<ST, A><<<grid, 256, 0, s>>>((ST*)out, ldo, ldo_in,            \
+      (const ST*)g, (const ST*)u, ldi, ldi_in, rg, (const ST*)bg,          \
+      (const ST*)bu, (const float*)rw, R, F)
+#define GLU_ACT(ST)                                   \
+  do {                                                \
+    if (act == 0) GLU(ST, 0);                         \
+    else if (act == 1) GLU(ST, 1);                    \
+    else GLU(ST, 2);                                  \
+  } while (0)
+  MIX_DISPATCH(dt, GLU_ACT(u16), GLU_ACT(float));
+#undef GLU_ACT
+#undef GLU
+  return af_last_err();
+}
+
+AF_EXPORT int afm_moe_route(void* idx, void* wts, void* wd, const void* z,
+                            const void* corr, int T, int E, int top,
+                            int n_groups, int keep, float scale,
+                            void* stream) {
+  if (T == 0) return 0;
+  if (E < 1 || top < 1 || top > E) return 9003;
+  if (n_groups > 0 && (E % n_groups != 0 || keep < 1)) return 9003;
+  const size_t sm = (size_t)(2 * E + (n_groups > 0 ? n_groups : 0)) *
+                    sizeof(float);
+  if (sm > 60000) return 9004;
+  moe_route_kernel<<<T, 64, sm, (hipStream_t)stream>>>(
+      (i32*)idx, (float*)wts, (float*)wd, (const float*)z, (const float*)corr,
+      E, top, n_groups, keep, scale);
+  return af_last_err();
+}
+
+AF_EXPORT int afm_moe_combine(void* y, const void* ys, const void* pos,
+                              const void* wts, const void* shared, int T,
+                              int top, int W, int dt, void* stream) {
+  if (T == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  MIX_DISPATCH(dt,
+      (moe_combine_kernel<u16><<<T, 256, 0, s>>>((float*)y, (const u16*)ys,
+          (const i32*)pos, (const float*)wts, (const u16*)shared, top, W)),
+      (moe_combine_kernel<float><<<T, 256, 0, s>>>((float*)y, (const float*)ys,
+          (const i32*)pos, (const float*)wts, (const float*)shared, top, W)));
   return af_last_err();
 }

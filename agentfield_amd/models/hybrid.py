@@ -25,6 +25,7 @@ the engine's scheduler hands out both.
 from __future__ import annotations
 
 import json
+import math
 from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Callable
@@ -119,6 +120,21 @@ class ReperaxConfig:
     def build_model(self, device="cpu", dtype=torch.bfloat16):
         return ReperaxForCausalLM(self, device=device, dtype=dtype)
 
+    def cache_layout(self) -> list:
+        """What every layer run keeps between steps (HybridCache)."""
+        out = []
+        for li, _p in self.runs:
+            ls = self.layers[li]
+            m = ls.gla if ls.kind == "parallel" else ls.ret
+            need = {"kv": None, "state": {
+                "shift": ((self.width,), "f32"),
+                "rec": ((m.heads, m.dim, m.vdim), "f32")}}
+            if ls.kind == "parallel":
+                a = ls.attn
+                need["kv"] = (a.kv_heads, a.dim, a.vdim)
+            out.append(need)
+        return out
+
     @staticmethod
     def from_json(c: dict, shape_of: Callable[[str], tuple] | None = None,
                   name: str = "reperax") -> "ReperaxConfig":
@@ -199,55 +215,57 @@ class ReperaxConfig:
 
 # ------------------------------------------------------------------ cache
 class HybridCache:
-    """Per-run storage for one engine: K/V pages for attention mixers
-    ([P, G, page, dk] / [P, G, page, dv] in the model dtype), fp32 recurrent
-    matrices [slots, H, dk, dv] and fp32 token-shift rows [slots, W] for
-    every run.  Page 0 and slot 0 are the engine's null page / null slot.
-    Nothing is cleared when a page or slot changes hands: a chunk that starts
-    at position 0 ignores the slot's content, and attention never reads a
-    position that the current owner has not written."""
+    """Per-run storage for one engine, built from a model's cache layout:
+    one entry per layer run (a looped layer counts once per pass) with
 
-    def __init__(self, cfg: ReperaxConfig, num_pages: int, page_size: int,
+      "kv":    (kv_heads, dk, dv) or None - K/V pages [P, G, page, dk] /
+               [P, G, page, dv] in the model dtype
+      "state": {name: (shape, "f32" | "model")} - per-sequence tensors
+               [slots, *shape] (recurrent matrices, token-shift rows,
+               convolution inputs, ...)
+
+    Pages live in `k[run]` / `v[run]`, state in `state[name][run]` (`rec` and
+    `shift` are the names the linear-recurrence layers use).  Page 0 and slot
+    0 are the engine's null page / null slot.  Nothing is cleared when a page
+    or slot changes hands: a chunk that starts at position 0 ignores the
+    slot's content, and attention never reads a position that the current
+    owner has not written."""
+
+    def __init__(self, layout: list, num_pages: int, page_size: int,
                  num_slots: int, device, dtype=torch.bfloat16):
         self.page_size, self.num_pages, self.num_slots = \
             page_size, num_pages, num_slots
-        self.k, self.v, self.rec, self.shift = {}, {}, {}, {}
-        for r, (li, _p) in enumerate(cfg.runs):
-            ls = cfg.layers[li]
-            self.shift[r] = torch.zeros(num_slots, cfg.width,
-                                        dtype=torch.float32, device=device)
-            if ls.kind == "parallel":
-                a, g = ls.attn, ls.gla
-                self.k[r] = torch.zeros(num_pages, a.kv_heads, page_size,
-                                        a.dim, dtype=dtype, device=device)
-                self.v[r] = torch.zeros(num_pages, a.kv_heads, page_size,
-                                        a.vdim, dtype=dtype, device=device)
-                self.rec[r] = torch.zeros(num_slots, g.heads, g.dim, g.vdim,
-                                          dtype=torch.float32, device=device)
-            else:
-                t = ls.ret
-                self.rec[r] = torch.zeros(num_slots, t.heads, t.dim, t.vdim,
-                                          dtype=torch.float32, device=device)
+        self.k, self.v, self.state = {}, {}, {}
+        for r, need in enumerate(layout):
+            kv = need.get("kv")
+            if kv is not None:
+                G, dk, dv = kv
+                self.k[r] = torch.zeros(num_pages, G, page_size, dk,
+                                        dtype=dtype, device=device)
+                self.v[r] = torch.zeros(num_pages, G, page_size, dv,
+                                        dtype=dtype, device=device)
+            for name, (shape, kind) in (need.get("state") or {}).items():
+                self.state.setdefault(name, {})[r] = torch.zeros(
+                    num_slots, *shape, device=device,
+                    dtype=torch.float32 if kind == "f32" else dtype)
+        self.rec = self.state.get("rec", {})
+        self.shift = self.state.get("shift", {})
 
     @staticmethod
-    def bytes_per_page(cfg: ReperaxConfig, page_size: int,
-                       itemsize: int = 2) -> int:
+    def bytes_per_page(layout: list, page_size: int, itemsize: int = 2) -> int:
         n = 0
-        for li, _p in cfg.runs:
-            ls = cfg.layers[li]
-            if ls.kind == "parallel":
-                n += ls.attn.kv_heads * page_size * \
-                    (ls.attn.dim + ls.attn.vdim) * itemsize
+        for need in layout:
+            if need.get("kv") is not None:
+                G, dk, dv = need["kv"]
+                n += G * page_size * (dk + dv) * itemsize
         return max(n, 1)
 
     @staticmethod
-    def bytes_per_slot(cfg: ReperaxConfig) -> int:
+    def bytes_per_slot(layout: list, itemsize: int = 2) -> int:
         n = 0
-        for li, _p in cfg.runs:
-            ls = cfg.layers[li]
-            n += cfg.width * 4
-            m = ls.gla if ls.kind == "parallel" else ls.ret
-            n += m.heads * m.dim * m.vdim * 4
+        for need in layout:
+            for shape, kind in (need.get("state") or {}).values():
+                n += math.prod(shape) * (4 if kind == "f32" else itemsize)
         return n
 
 
@@ -446,11 +464,11 @@ class ReperaxForCausalLM(nn.Module):
     # -- engine interface ---------------------------------------------------
     def make_cache(self, num_pages: int, page_size: int, num_slots: int,
                    device, dtype):
-        return HybridCache(self.cfg, num_pages, page_size, num_slots, device,
-                           dtype)
+        return HybridCache(self.cfg.cache_layout(), num_pages, page_size,
+                           num_slots, device, dtype)
 
     def cache_bytes_per_page(self, page_size: int) -> int:
-        return HybridCache.bytes_per_page(self.cfg, page_size,
+        return HybridCache.bytes_per_page(self.cfg.cache_layout(), page_size,
                                           self.embed.element_size())
 
     def forward(self, ids, positions, cache: HybridCache, md,

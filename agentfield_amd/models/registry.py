@@ -73,6 +73,13 @@ def _load_reperax(path, device="cpu", dtype=None, **kw):
                         max_position=kw.get("max_position"))
 
 
+def _load_zudisun(path, device="cpu", dtype=None, **kw):
+    from .zudisun import load_zudisun
+    return load_zudisun(path, device=device, dtype=dtype,
+                        max_position=kw.get("max_position"))
+
+
 register_architecture(["LlamaForCausalLM", "MistralForCausalLM",
                        "MixtralForCausalLM"], _load_llama)
 register_architecture("Reperax", _load_reperax)
+register_architecture("Zudisun", _load_zudisun)

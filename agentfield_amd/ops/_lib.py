@@ -82,53 +82,93 @@ def _declare(l: ctypes.CDLL) -> None:
         getattr(l, fn).restype = ctypes.c_int
 
 
-_MIX_PATH = Path(__file__).resolve().parent.parent / "libafmix.so"
-
-
-@functools.lru_cache(maxsize=1)
-def mixlib() -> ctypes.CDLL:
-    """The sequence-mixer kernel group (ops/seqmix.py).  Unlike the main
-    library it is compiled on first use when missing or older than its
-    sources — on a GPU box too — so a fresh checkout serving a hybrid model
-    builds exactly this group and nothing else."""
-    from agentfield_amd.build import build_mix
+@functools.lru_cache(maxsize=None)
+def mixgroup(group: str) -> ctypes.CDLL:
+    """One sequence-mixer kernel group (build.MIX_GROUPS).  Unlike the main
+    library a group is compiled on first use when missing or older than its
+    sources - on a GPU box too - so a fresh checkout serving a hybrid model
+    builds exactly the groups that model calls and nothing else."""
+    from agentfield_amd.build import MIX_GROUPS, build_mix
+    path = MIX_GROUPS[group][0]
     try:
-        build_mix(verbose=False)
+        build_mix(verbose=False, group=group)
     except Exception as e:
-        if not _MIX_PATH.exists():
-            raise AfOpsError(f"libafmix.so could not be built: {e}") from e
-    cdll = ctypes.CDLL(str(_MIX_PATH))
-    _declare_mix(cdll)
+        if not path.exists():
+            raise AfOpsError(f"{path.name} could not be built: {e}") from e
+    cdll = ctypes.CDLL(str(path))
+    for name, args in _MIX_SIGS[group].items():
+        fn = getattr(cdll, name)
+        fn.argtypes = args
+        fn.restype = ctypes.c_int
     return cdll
 
 
-def _declare_mix(l: ctypes.CDLL) -> None:
+class _MixLib:
+    """Resolves an afm_* entry point to its kernel group on first use."""
+
+    def __getattr__(self, name):
+        for group, sigs in _MIX_SIGS.items():
+            if name in sigs:
+                fn = getattr(mixgroup(group), name)
+                setattr(self, name, fn)
+                return fn
+        raise AttributeError(name)
+
+
+_MIXLIB = _MixLib()
+
+
+def mixlib() -> _MixLib:
+    return _MIXLIB
+
+
+def _mix_sigs() -> dict:
     p, i, i64, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
-    sig = {
-        "afm_embed": [p, p, p, p, i, i, i, p],
-        "afm_add_rows": [p, p, p, i, i, p],
-        "afm_dual_norm_shift": [p, p, p, p, p, p, p, p, p, p, p, p, p, f,
-                                i, i, i, p],
-        "afm_scatter_state": [p, p, p, p, i, i, p],
-        "afm_norm_rows": [p, p, p, p, f, i, i, i, i, p],
-        "afm_headnorm_gate": [p, p, p, p, f, i, i, i, i64, i, p],
-        "afm_polynorm": [p, p, p, f, i, i, i64, i, p],
-        "afm_gated_residual": [p, p, f, p, f, p, i64, p, p, p, i64, p,
-                               i, i, i, p],
-        "afm_softcap": [p, p, f, i64, i, p],
-        "afm_qk_norm_cache": [p, p, p, p, p, p, p, p, p, f, i, i, i, i, i, i,
-                              i, i, i64, i64, i64, i, p],
-        "afm_masked_attention": [p, p, p, p, p, p, p, f, i, i, i, i, i, i, i,
-                                 i, i, i64, i, p, p, i, p],
-        "afm_attn_prefill_mfma": [p, p, p, p, p, p, p, p, p, f, i, i, i, i, i,
-                                  i, i, i, i, i64, p],
-        "afm_linear_scan": [p, p, p, p, p, p, p, p, p, p, p, p, p, f, f, f,
-                            i, i, i, i, i, i64, i64, i64, i64, i, p],
+    return {
+        "glue": {
+            "afm_embed": [p, p, p, p, i, i, i, p],
+            "afm_add_rows": [p, p, p, i, i, p],
+            "afm_dual_norm_shift": [p, p, p, p, p, p, p, p, p, p, p, p, p, f,
+                                    i, i, i, p],
+            "afm_scatter_state": [p, p, p, p, i, i, p],
+            "afm_norm_rows": [p, p, p, p, f, i, i, i, i, p],
+            "afm_headnorm_gate": [p, p, p, p, f, i, i, i, i64, i, p],
+            "afm_polynorm": [p, p, p, f, i, i, i64, i, p],
+            "afm_gated_residual": [p, p, f, p, f, p, i64, p, p, p, i64, p,
+                                   i, i, i, p],
+            "afm_softcap": [p, p, f, i64, i, p],
+            "afm_cast_rows": [p, p, i64, i, p],
+            "afm_norm_residual": [p, p, p, i64, i, p, p, f, i, i, i, p],
+            "afm_glu": [p, i64, i64, p, p, i64, i64, i, p, p, p, i64, i, i,
+                        i, p],
+            "afm_moe_route": [p, p, p, p, p, i, i, i, i, i, f, p],
+            "afm_moe_combine": [p, p, p, p, p, i, i, i, i, p],
+        },
+        "seq": {
+            "afm_qk_norm_cache": [p, p, p, p, p, p, p, p, p, f, i, i, i, i, i,
+                                  i, i, i, i64, i64, i64, i, p],
+            "afm_masked_attention": [p, p, p, p, p, p, p, f, i, i, i, i, i, i,
+                                     i, i, i, i64, i, p, p, i, p],
+            "afm_attn_prefill_mfma": [p, p, p, p, p, p, p, p, p, f, i, i, i, i,
+                                      i, i, i, i, i, i64, p],
+            "afm_linear_scan": [p, p, p, p, p, p, p, p, p, p, p, p, p, f, f, f,
+                                i, i, i, i, i, i64, i64, i64, i64, i, p],
+        },
+        "ssm": {
+            "afm_causal_conv": [p, p, i64, p, p, p, p, p, p, p, i, i, i, i, i,
+                                i, p],
+            "afm_selective_scan": [p, p, p, p, p, p, i64, p, i64, p, p, p, p,
+                                   p, i, i, i, i, p],
+            "afm_qk_unit_cache": [p, p, i64, p, i64, p, i64, p, i64, f, p, p,
+                                  p, p, f, f, i, i, i, i, i, i, i, i, p],
+            "afm_sigmoid_attention": [p, p, p, p, p, p, p, p, p, p, i, i, p, p,
+                                      p, i64, f, i, i, i, i, i, i, i, i, i, i,
+                                      p],
+        },
     }
-    for name, args in sig.items():
-        fn = getattr(l, name)
-        fn.argtypes = args
-        fn.restype = ctypes.c_int
+
+
+_MIX_SIGS = _mix_sigs()
 
 
 def cur_stream() -> ctypes.c_void_p:

@@ -11,7 +11,7 @@ Conventions shared by every op here:
     chunk's first row), row_seq [T] i32 (sequence index of every row),
     state_slots [B] i32 (per-sequence state slot), a decode step being the
     special case of one row per sequence
-  * CUDA (=HIP) tensors run the gfx950 kernels in libafmix.so, CPU tensors a
+  * CUDA (=HIP) tensors run the gfx950 kernels of the mixer kernel groups, CPU tensors a
     vectorised torch path used by CPU tests
 
 The recurrences are evaluated strictly token by token in fp32, so results
@@ -19,6 +19,7 @@ do not depend on where a prompt was cut into chunks.
 """
 from __future__ import annotations
 
+import ctypes
 import math
 import os
 
@@ -467,3 +468,385 @@ def matmul(x: torch.Tensor, w: torch.Tensor,
         from . import linear_skinny
         return linear_skinny(x, w)
     return x @ w.t()
+
+
+# =====================================================================
+# Ops of post-norm hybrid decoders: sublayers read the residual itself, a
+# norm sits on each sublayer's output; selective state-space mixer, sigmoid
+# attention with distance bias and head mixing, gated units, sigmoid router.
+# =====================================================================
+def cast_rows(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """The fp32 residual in the storage dtype (itself when that is fp32)."""
+    if x.dtype == dtype:
+        return x
+    if not _gpu(x):
+        return x.to(dtype)
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    rc = _L().afm_cast_rows(_lib.ptr(out), _lib.ptr(x), x.numel(), _code(out),
+                            _lib.cur_stream())
+    _lib.check(rc, "afm_cast_rows")
+    return out
+
+
+def norm_residual(x: torch.Tensor, y: torch.Tensor,
+                  bias: torch.Tensor | None, w: torch.Tensor, eps: float,
+                  dtype: torch.dtype) -> torch.Tensor:
+    """In place on the fp32 residual: u = y (+ bias); x += u / rms(u) * w.
+    y [T, W] is in the storage dtype or fp32.  Returns the new residual in
+    `dtype` (x itself for fp32), the next sublayer's input."""
+    T, W = x.shape
+    if not _gpu(x):
+        u = y.float()
+        if bias is not None:
+            u = u + bias.float()
+        x += u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        return x.to(dtype) if dtype != torch.float32 else x
+    h = None if dtype == torch.float32 else \
+        torch.empty(T, W, dtype=dtype, device=x.device)
+    rc = _L().afm_norm_residual(
+        _lib.ptr(x), _lib.ptr(h), _lib.ptr(y), _rowstride(y),
+        1 if y.dtype == torch.float32 else 0, _lib.ptr(bias), _lib.ptr(w),
+        float(eps), T, W, _code(w), _lib.cur_stream())
+    _lib.check(rc, "afm_norm_residual")
+    return x if h is None else h
+
+
+GLU_ACTS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+
+
+def _act(name: str, a: torch.Tensor) -> torch.Tensor:
+    if name == "silu":
+        return a * torch.sigmoid(a)
+    if name == "relu":
+        return torch.relu(a)
+    return 0.5 * a * (1.0 + torch.tanh(
+        0.7978845608028654 * (a + 0.044715 * a ** 3)))
+
+
+def glu(gu: torch.Tensor, F: int, act: str,
+        bias: torch.Tensor | None = None, units: int = 1,
+        row_weight: torch.Tensor | None = None,
+        out: torch.Tensor | None = None) -> torch.Tensor:
+    """act(gate + bg) * (up + bu) (* row_weight) for `units` gated units
+    laid side by side in every row of gu [T, >= units*2F], unit e being
+    [gate_e (F) | up_e (F)].  bias [2F] = [bg | bu] (units == 1 only);
+    row_weight [T, units] fp32.  Writes out [T, >= units*F] (allocated
+    [T, units*F] when not given)."""
+    T = gu.shape[0]
+    if out is None:
+        out = torch.empty(T, units * F, dtype=gu.dtype, device=gu.device)
+    if not _gpu(gu):
+        v = gu[:, :units * 2 * F].float().reshape(T, units, 2 * F)
+        g, u = v[..., :F], v[..., F:]
+        if bias is not None:
+            g, u = g + bias[:F].float(), u + bias[F:].float()
+        o = _act(act, g) * u
+        if row_weight is not None:
+            o = o * row_weight.float().reshape(T, units, 1)
+        out[:, :units * F] = o.reshape(T, units * F).to(out.dtype)
+        return out
+    rc = _L().afm_glu(
+        _lib.ptr(out), _rowstride(out), F, _lib.ptr(gu),
+        ctypes.c_void_p(gu.data_ptr() + F * gu.element_size()),
+        _rowstride(gu), 2 * F, units,
+        _lib.ptr(bias[:F]) if bias is not None else None,
+        _lib.ptr(bias[F:]) if bias is not None else None,
+        _lib.ptr(row_weight), T * units, F, GLU_ACTS[act], _code(gu),
+        _lib.cur_stream())
+    _lib.check(rc, "afm_glu")
+    return out
+
+
+def moe_route(z: torch.Tensor, correction: torch.Tensor | None, top: int,
+              n_groups: int = 0, keep: int = 0, scale: float = 1.0,
+              dense: bool = False):
+    """Sigmoid router with score correction and group-limited top-k.
+
+    z [T, E] fp32 logits; s = sigmoid(z); choice = s + correction.  With
+    n_groups > 0 the experts form equal groups of neighbours, a group scores
+    the sum of its two largest choice scores and only experts of the `keep`
+    best groups can be chosen.  The `top` largest choice scores win; weights
+    = s / (sum of the chosen s + 1e-20) * scale.  Returns (idx [T, top] i32,
+    weights [T, top] fp32, dense weights [T, E] fp32 or None)."""
+    T, E = z.shape
+    if not _gpu(z):
+        s = torch.sigmoid(z.float())
+        choice = s + correction.float() if correction is not None else s.clone()
+        if n_groups > 0 and keep < n_groups:
+            size = E // n_groups
+            gs = choice.view(T, n_groups, size).topk(min(2, size), -1)[0].sum(-1)
+            kept = torch.zeros(T, n_groups, dtype=torch.bool)
+            kept.scatter_(1, gs.topk(keep, -1)[1], True)
+            choice = choice.masked_fill(
+                ~kept.repeat_interleave(size, dim=1), -math.inf)
+        idx = choice.topk(top, -1)[1]
+        w = s.gather(1, idx)
+        w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+        wd = None
+        if dense:
+            wd = torch.zeros(T, E).scatter_(1, idx, w)
+        return idx.to(torch.int32), w, wd
+    z = z.contiguous()
+    idx = torch.empty(T, top, dtype=torch.int32, device=z.device)
+    w = torch.empty(T, top, dtype=torch.float32, device=z.device)
+    wd = torch.empty(T, E, dtype=torch.float32, device=z.device) \
+        if dense else None
+    rc = _L().afm_moe_route(_lib.ptr(idx), _lib.ptr(w), _lib.ptr(wd),
+                            _lib.ptr(z), _lib.ptr(correction), T, E, top,
+                            int(n_groups), int(keep), float(scale),
+                            _lib.cur_stream())
+    _lib.check(rc, "afm_moe_route")
+    return idx, w, wd
+
+
+def moe_combine(ys: torch.Tensor, pos: torch.Tensor, weights: torch.Tensor,
+                shared: torch.Tensor | None) -> torch.Tensor:
+    """y[t] = sum_r weights[t, r] * ys[pos[t*top + r]] (+ shared[t]), fp32,
+    summed in the order r = 0..top-1.  ys [T*top, W] holds the experts'
+    outputs in expert-sorted order, pos [T*top] i32 the place of every
+    (token, choice) in it."""
+    T, top = weights.shape
+    W = ys.shape[1]
+    if not _gpu(ys):
+        y = (ys.float()[pos.long()].view(T, top, W)
+             * weights.float()[:, :, None])
+        out = shared.float().clone() if shared is not None else \
+            torch.zeros(T, W)
+        for r in range(top):
+            out += y[:, r]
+        return out
+    out = torch.empty(T, W, dtype=torch.float32, device=ys.device)
+    rc = _L().afm_moe_combine(_lib.ptr(out), _lib.ptr(ys), _lib.ptr(pos),
+                              _lib.ptr(weights), _lib.ptr(shared), T, top, W,
+                              _code(ys), _lib.cur_stream())
+    _lib.check(rc, "afm_moe_combine")
+    return out
+
+
+# ------------------------------------------------- selective state space
+def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None,
+                state: torch.Tensor, md, silu: bool = True) -> torch.Tensor:
+    """Depthwise causal convolution over packed chunks: out[t, c] = act(b[c]
+    + sum_j w[c, j] x[t - (taps-1-j), c]), the last column weighing the
+    current token.  Inputs from before a chunk come from the sequence's slot
+    of `state` [slots, taps-1, C] (storage dtype, oldest first), inputs
+    before position 0 are zero; afterwards the slot holds the sequence's last
+    taps-1 inputs.  x [T, C] may be a strided view."""
+    T, C = x.shape
+    taps = w.shape[1]
+    B = md.q_start.numel()
+    if not _gpu(x):
+        out = torch.empty(T, C, dtype=torch.float32)
+        cu, qs, sl = (md.cu_seqlens.tolist(), md.q_start.tolist(),
+                      md.state_slots.tolist())
+        wf = w.float()
+        for b in range(B):
+            r0, r1 = cu[b], cu[b + 1]
+            if r1 == r0:
+                continue
+            hist = state[sl[b]].float() if qs[b] > 0 else \
+                torch.zeros(taps - 1, C)
+            cat = torch.cat([hist, x[r0:r1].float()], 0)
+            acc = torch.zeros(r1 - r0, C)
+            if bias is not None:
+                acc += bias.float()
+            for j in range(taps):
+                acc += wf[:, j] * cat[j:j + r1 - r0]
+            out[r0:r1] = acc
+            if taps > 1:
+                state[sl[b]] = cat[-(taps - 1):].to(state.dtype)
+        if silu:
+            out = out * torch.sigmoid(out)
+        return out.to(x.dtype)
+    out = torch.empty(T, C, dtype=x.dtype, device=x.device)
+    rc = _L().afm_causal_conv(
+        _lib.ptr(out), _lib.ptr(x), _rowstride(x), _lib.ptr(w),
+        _lib.ptr(bias), _lib.ptr(state), _lib.ptr(md.row_seq),
+        _lib.ptr(md.cu_seqlens), _lib.ptr(md.q_start),
+        _lib.ptr(md.state_slots), T, B, C, taps, 1 if silu else 0, _code(x),
+        _lib.cur_stream())
+    _lib.check(rc, "afm_causal_conv")
+    return out
+
+
+def selective_scan(x: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor,
+                   bc: torch.Tensor, N: int, z: torch.Tensor,
+                   A: torch.Tensor, D: torch.Tensor, state: torch.Tensor,
+                   md) -> torch.Tensor:
+    """Selective scan, token by token in fp32, per channel c and state n:
+
+        d = softplus(dt[t, c] + dt_bias[c])
+        S[c, n] <- exp(d A[c, n]) S[c, n] + d x[t, c] B[t, n]
+        y[t, c] = (sum_n S[c, n] C[t, n] + D[c] x[t, c]) * silu(z[t, c])
+
+    bc [T, >= 2N] holds [B | C] per row (may be a strided view, as may z);
+    A [C, N], D [C] fp32; state [slots, C, N] fp32 is read unless the chunk
+    starts at position 0 and written after the chunk's last row."""
+    T, C = x.shape
+    B = md.q_start.numel()
+    if not _gpu(x):
+        d = torch.nn.functional.softplus(dt.float() + dt_bias.float(),
+                                         threshold=20.0)
+        xf, zf = x.float(), z.float()
+        Bm, Cm = bc[:, :N].float(), bc[:, N:2 * N].float()
+        y = torch.empty(T, C, dtype=torch.float32)
+        cu, qs, sl = (md.cu_seqlens.tolist(), md.q_start.tolist(),
+                      md.state_slots.tolist())
+        for b in range(B):
+            if cu[b + 1] == cu[b]:
+                continue
+            S = state[sl[b]].clone() if qs[b] > 0 else torch.zeros(C, N)
+            for t in range(cu[b], cu[b + 1]):
+                S = torch.exp(d[t][:, None] * A) * S + \
+                    (d[t] * xf[t])[:, None] * Bm[t][None]
+                y[t] = S @ Cm[t] + D * xf[t]
+            state[sl[b]] = S
+        return (y * zf * torch.sigmoid(zf)).to(x.dtype)
+    out = torch.empty(T, C, dtype=x.dtype, device=x.device)
+    rc = _L().afm_selective_scan(
+        _lib.ptr(out), _lib.ptr(state), _lib.ptr(x.contiguous()),
+        _lib.ptr(dt.contiguous()), _lib.ptr(dt_bias), _lib.ptr(bc),
+        _rowstride(bc), _lib.ptr(z), _rowstride(z), _lib.ptr(A), _lib.ptr(D),
+        _lib.ptr(md.cu_seqlens), _lib.ptr(md.q_start),
+        _lib.ptr(md.state_slots), B, C, N, _code(x), _lib.cur_stream())
+    _lib.check(rc, "afm_selective_scan")
+    return out
+
+
+# ------------------------------------------------------ sigmoid attention
+def distance_buckets(rows: int, dmax: float) -> torch.Tensor:
+    """Bucket of every distance below dmax for a learned distance bias with
+    `rows` rows: n itself below rows/2, then logarithmic steps that reach the
+    last row at dmax; distances from dmax on all take the last row (callers
+    clamp).  i32 [ceil(dmax)], evaluated in double precision on the host."""
+    half = rows // 2
+    out = []
+    for n in range(max(int(math.ceil(dmax)), half)):
+        if n < half:
+            out.append(n)
+            continue
+        v = math.log(n / half) / math.log(dmax / half) * (rows - half)
+        out.append(min(rows - 1, half + int(math.floor(v + 1e-9))))
+    return torch.tensor(out, dtype=torch.int32)
+
+
+def qk_unit_cache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                  heads: int, kv_heads: int, eps: float,
+                  kcache: torch.Tensor, vcache: torch.Tensor,
+                  slots: torch.Tensor, positions: torch.Tensor,
+                  temp_coef: float = 0.0, temp_every: int = 0,
+                  v_first: torch.Tensor | None = None,
+                  lam: float = 0.0) -> torch.Tensor:
+    """Per head: q and k divided by their root mean square (no weight); q
+    times 1 + temp_coef * ln(floor((p+1)/temp_every) + 1) at position p
+    (temp_every 0: no temperature); v <- (1-lam) v + lam v_first when v_first
+    is given.  k and v are appended to the paged caches at `slots`.  Inputs
+    may be strided views.  Returns q, contiguous [T, H*dk]."""
+    T = q.shape[0]
+    H, G = heads, kv_heads
+    dk = q.shape[1] // H
+    dv = v.shape[1] // G
+    page = kcache.shape[2]
+    if not _gpu(q):
+        qf = q.float().reshape(T, H, dk)
+        kf = k.float().reshape(T, G, dk)
+        qf = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps)
+        kf = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps)
+        if temp_every > 0:
+            steps = torch.div(positions + 1, temp_every,
+                              rounding_mode="floor").float()
+            qf = qf * (1.0 + temp_coef * torch.log(steps + 1.0))[:, None, None]
+        vf = v.float()
+        if v_first is not None:
+            vf = (1.0 - lam) * vf + lam * v_first.float()
+        pg = torch.div(slots, page, rounding_mode="floor")
+        off = slots - pg * page
+        kcache[pg, :, off] = kf.to(kcache.dtype)
+        vcache[pg, :, off] = vf.reshape(T, G, dv).to(vcache.dtype)
+        return qf.reshape(T, H * dk).to(q.dtype)
+    out = torch.empty(T, H * dk, dtype=q.dtype, device=q.device)
+    rc = _L().afm_qk_unit_cache(
+        _lib.ptr(out), _lib.ptr(q), _rowstride(q), _lib.ptr(k), _rowstride(k),
+        _lib.ptr(v), _rowstride(v), _lib.ptr(v_first),
+        _rowstride(v_first) if v_first is not None else 0, float(lam),
+        _lib.ptr(kcache), _lib.ptr(vcache), _lib.ptr(slots),
+        _lib.ptr(positions), float(eps), float(temp_coef), int(temp_every),
+        T, H, G, dk, dv, page, _code(q), _lib.cur_stream())
+    _lib.check(rc, "afm_qk_unit_cache")
+    return out
+
+
+def sigmoid_attention(q: torch.Tensor, kcache: torch.Tensor,
+                      vcache: torch.Tensor, md, positions: torch.Tensor,
+                      scale: float, heads: int,
+                      rel: torch.Tensor | None = None,
+                      buckets: torch.Tensor | None = None,
+                      talk: torch.Tensor | None = None,
+                      head_bias: torch.Tensor | None = None,
+                      gate: torch.Tensor | None = None,
+                      window: int = 0) -> torch.Tensor:
+    """Attention with un-normalised sigmoid weights over the paged cache.
+    For the row at position i and every key j <= i (and j > i - window when
+    window > 0), per head h:
+
+        s_h = q_h . k_g(h) * scale + rel[bucket(i - j), h]
+        m_h = sum_g talk[h, g] s_g                 (all heads of the pair)
+        o_h = sum_j sigmoid(m_h + head_bias[h]) v_j,   o_h *= sigmoid(gate_h)
+
+    rel [rows, H], talk [H, H], head_bias [H] fp32 (each optional); buckets
+    i32 from distance_buckets (distances past its end use the last row);
+    gate [T, H] logits in the storage dtype (may be a strided view).
+    q [T, H*dk] -> [T, H*dv]."""
+    T = q.shape[0]
+    _, G, page, dk = kcache.shape
+    dv = vcache.shape[3]
+    H = heads
+    RB = rel.shape[0] if rel is not None else 0
+    if not _gpu(q):
+        out = torch.zeros(T, H, dv, dtype=torch.float32)
+        qf = q.float().view(T, H, dk)
+        bt = md.block_table.long()
+        rs = md.row_seq.tolist()
+        pos = positions.tolist()
+        for t in range(T):
+            i = pos[t]
+            lo = max(0, i - window + 1) if window > 0 else 0
+            js = torch.arange(lo, i + 1)
+            pg = bt[rs[t]][js // page]
+            kk = kcache[pg, :, js % page].float()      # [n, G, dk]
+            vv = vcache[pg, :, js % page].float()
+            kk = kk.repeat_interleave(H // G, dim=1)
+            vv = vv.repeat_interleave(H // G, dim=1)
+            s = torch.einsum("nhd,hd->hn", kk, qf[t]) * scale
+            if rel is not None:
+                dist = (i - js).clamp(max=buckets.numel())
+                bk = torch.cat([buckets.long(),
+                                torch.tensor([RB - 1])])[dist]
+                s = s + rel.float()[bk].t()
+            if talk is not None:
+                s = talk.float() @ s
+            if head_bias is not None:
+                s = s + head_bias.float()[:, None]
+            out[t] = torch.einsum("hn,nhd->hd", torch.sigmoid(s), vv)
+        if gate is not None:
+            out = out * torch.sigmoid(gate.float())[:, :, None]
+        return out.view(T, H * dv).to(q.dtype)
+    out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+    # few rows and a long reach: cut each row's keys over several workgroups
+    reach = md.block_table.shape[1] * page
+    if window > 0:
+        reach = min(reach, window)
+    nsplit = max(1, min(16, 1024 // max(1, T), reach // 256))
+    part = torch.empty(T, nsplit, H * dv, dtype=torch.float32,
+                       device=q.device)
+    rc = _L().afm_sigmoid_attention(
+        _lib.ptr(out), _lib.ptr(part), _lib.ptr(q), _lib.ptr(kcache),
+        _lib.ptr(vcache), _lib.ptr(md.block_table), _lib.ptr(md.row_seq),
+        _lib.ptr(positions), _lib.ptr(rel), _lib.ptr(buckets),
+        buckets.numel() if buckets is not None else 0, RB, _lib.ptr(talk),
+        _lib.ptr(head_bias), _lib.ptr(gate),
+        _rowstride(gate) if gate is not None else 0, float(scale), T, H, G,
+        dk, dv, page, md.block_table.shape[1], nsplit, int(window), _code(q),
+        _lib.cur_stream())
+    _lib.check(rc, "afm_sigmoid_attention")
+    return out
