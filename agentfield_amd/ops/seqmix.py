@@ -644,7 +644,7 @@ def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None,
             r0, r1 = cu[b], cu[b + 1]
             if r1 == r0:
                 continue
-            hist = state[sl[b]].float() if qs[b] > 0 else \
+            hist = state[sl[b]][:taps - 1].float() if qs[b] > 0 else \
                 torch.zeros(taps - 1, C)
             cat = torch.cat([hist, x[r0:r1].float()], 0)
             acc = torch.zeros(r1 - r0, C)
@@ -654,7 +654,7 @@ def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None,
                 acc += wf[:, j] * cat[j:j + r1 - r0]
             out[r0:r1] = acc
             if taps > 1:
-                state[sl[b]] = cat[-(taps - 1):].to(state.dtype)
+                state[sl[b]][:taps - 1] = cat[-(taps - 1):].to(state.dtype)
         if silu:
             out = out * torch.sigmoid(out)
         return out.to(x.dtype)

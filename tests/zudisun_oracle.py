@@ -209,3 +209,79 @@ def forward(tokens, cfg, P, keep_layers=False):
             layers.append(x.clone())
     logits = rms_norm(x, P["final.norm"], eps) @ _f(P["head"]).t()
     return (logits, layers) if keep_layers else logits
+
+
+# ------------------------------------------------------------ test weights
+def random_weights(cfg, seed, dtype=torch.float32):
+    """Checkpoint-named random tensors for a config (values rounded to
+    `dtype`), at scales that keep every branch alive: step sizes spread over
+    two decades, distinct distance-bias rows, a head-mixing matrix away from
+    the identity, corrections that change which experts win."""
+    g = torch.Generator().manual_seed(seed)
+
+    def r(*shape, std=1.0, mean=0.0):
+        return (torch.randn(*shape, generator=g) * std + mean).to(dtype)
+    W, V = cfg["width"], cfg["vocab"]
+    P = {"embed": r(V, W), "head": r(V, W, std=W ** -0.5),
+         "final.norm": r(W, std=0.2, mean=1.0)}
+    for i, lc in enumerate(cfg["layers"]):
+        pre, m = f"l{i}.mix.", lc["mixer"]
+        P[f"l{i}.norm1"] = r(W, std=0.2, mean=1.0)
+        if lc["type"] == "mamba1":
+            C, N, R, K = m["inner"], m["state"], m["dt_rank"], m["conv"]
+            P[pre + "in"] = r(2 * C, W, std=W ** -0.5)
+            P[pre + "conv"] = r(C, K, std=K ** -0.5)
+            P[pre + "conv.b"] = r(C, std=0.2)
+            P[pre + "x"] = r(R + 2 * N, C, std=C ** -0.5)
+            P[pre + "dt"] = r(C, R, std=R ** -0.5)
+            P[pre + "dt.b"] = r(C, std=1.5, mean=-2.0)
+            P[pre + "A_log"] = torch.log(
+                torch.rand(C, N, generator=g) * 4 + 0.05).to(dtype)
+            P[pre + "D"] = r(C, std=0.5, mean=1.0)
+            P[pre + "o"] = r(W, C, std=C ** -0.5)
+        else:
+            H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            P[pre + "q"] = r(H * dk, W, std=W ** -0.5)
+            P[pre + "k"] = r(G * dk, W, std=W ** -0.5)
+            P[pre + "v"] = r(G * dv, W, std=W ** -0.5)
+            P[pre + "g"] = r(H, W, std=W ** -0.5)
+            P[pre + "o"] = r(W, H * dv, std=(H * dv) ** -0.5)
+            P[pre + "rel"] = r(m.get("bias_rows", 32), H, std=0.7)
+            P[pre + "talk"] = (torch.eye(H) + torch.randn(H, H, generator=g)
+                               * 0.4).to(dtype)
+            P[pre + "pb"] = r(H, std=0.5, mean=-2.0)
+            P[pre + "vmix"] = torch.tensor(0.35).to(dtype)
+        mlp = lc.get("mlp")
+        if mlp is None:
+            continue
+        fp = f"l{i}.mlp."
+        P[f"l{i}.norm2"] = r(W, std=0.2, mean=1.0)
+
+        def unit(p, F, bias):
+            P[p + "gate"] = r(F, W, std=W ** -0.5)
+            P[p + "up"] = r(F, W, std=W ** -0.5)
+            P[p + "down"] = r(W, F, std=F ** -0.5)
+            if bias:
+                P[p + "gate.b"], P[p + "up.b"] = r(F, std=0.3), r(F, std=0.3)
+                P[p + "down.b"] = r(W, std=0.3)
+        if mlp["kind"] == "dense":
+            unit(fp, mlp["ff"], True)
+        else:
+            E = mlp["router"]["experts"]
+            for e in range(E):
+                unit(f"{fp}e{e}.", mlp["expert"]["ff"], False)
+            if mlp.get("shared"):
+                unit(fp + "shared.", mlp["shared"]["ff"], False)
+            P[fp + "router"] = r(E, W, std=2.0 * W ** -0.5)
+            P[fp + "correction"] = r(E, std=0.6, mean=-0.4)
+    return P
+
+
+def greedy(tokens, n, cfg, P):
+    """n greedy continuation tokens of a prompt."""
+    toks, out = list(tokens), []
+    for _ in range(n):
+        nxt = int(forward(toks, cfg, P)[-1].argmax())
+        out.append(nxt)
+        toks.append(nxt)
+    return out
