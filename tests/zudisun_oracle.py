@@ -272,7 +272,7 @@ def random_weights(cfg, seed, dtype=torch.float32):
                 unit(f"{fp}e{e}.", mlp["expert"]["ff"], False)
             if mlp.get("shared"):
                 unit(fp + "shared.", mlp["shared"]["ff"], False)
-            P[fp + "router"] = r(E, W, std=2.0 * W ** -0.5)
+            P[fp + "router"] = r(E, W, std=0.5 * W ** -0.5)
             P[fp + "correction"] = r(E, std=0.6, mean=-0.4)
     return P
 
