@@ -80,11 +80,13 @@ def parse_args():
     p.add_argument("--family-compare", action="store_true",
                    help="instead of the default workload: engine-level "
                         "prefill and decode token throughput of the hybrid "
-                        "(Reperax) family beside the Llama family at equal "
-                        "width / ff / depth, random weights; one JSON line "
-                        "per model and phase (single GPU)")
+                        "families (Reperax, Zudisun) beside each other and "
+                        "the Llama family at equal width / ff / depth, "
+                        "random weights; one JSON line per model and phase "
+                        "(single GPU)")
     p.add_argument("--compare-pairs", default="reperax-1b:debug-1b",
-                   help="comma list of hybrid:llama config-name pairs")
+                   help="comma list of colon-joined config names measured "
+                        "side by side, e.g. zudisun-1b:reperax-1b:debug-1b")
     p.add_argument("--cp-workers", type=int, default=0,
                    help="control-plane worker processes (0 = auto)")
     return p.parse_args()

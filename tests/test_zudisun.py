@@ -598,17 +598,36 @@ def test_greedy_generation_through_scheduler(device, dtype):
     outs = eng.generate(prompts, SamplingParams(max_tokens=12,
                                                 temperature=0.0,
                                                 ignore_eos=True))
+    # the GPU sampler reads logits rounded to bf16, so near-ties may fall
+    # either way: every emitted token must be (all but) the oracle's best
+    # given the tokens emitted before it
+    slack = 0.35 if dtype == torch.bfloat16 else \
+        (0.03 if device == "cuda" else 1e-3)
     for p, o in zip(prompts, outs):
-        if dtype == torch.float32:
-            assert o == orc.greedy(p, 12, cj, w)
-        else:
-            # bf16: every emitted token is (near) the best of the oracle's
-            # logits given the tokens emitted so far
-            toks = list(p)
-            for t in o:
-                lg = orc.forward(toks, cj, w)[-1]
-                assert float(lg.max() - lg[t]) < 0.25 * float(lg.std())
-                toks.append(t)
+        assert len(o) == 12
+        want = orc.forward(p + o, cj, w)
+        for i, tok in enumerate(o):
+            row = want[len(p) + i - 1]
+            assert row[tok] >= row.max() - slack, (len(p), i)
+    assert eng.state_slots.num_free == 4   # all slots given back
+
+
+def test_scheduler_preemption_restarts_state():
+    """Running out of pages preempts a sequence; on re-admission it
+    recomputes from position 0 in whatever slot is free and still produces
+    the oracle's greedy tokens."""
+    cj = cfg_degenerate()
+    eng, w = build(cj, "cpu", torch.float32, seed=17, page=4, pages=9,
+                   live=3, paced=False)
+    prompts = [tokens_for(cj, 6, 40 + i) for i in range(3)]
+    outs = eng.generate(prompts, SamplingParams(max_tokens=10,
+                                                ignore_eos=True))
+    assert eng.sched.n_preempted > 0
+    for p, o in zip(prompts, outs):
+        want = orc.forward(p + o, cj, w)
+        for i, tok in enumerate(o):
+            row = want[len(p) + i - 1]
+            assert row[tok] >= row.max() - 1e-3
 
 
 def test_config_round_trip_and_registry(tmp_path):
