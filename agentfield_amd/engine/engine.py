@@ -949,7 +949,15 @@ class LLMEngine:
             return entry
         nsplit = choose_nsplit(bs, self.cfg.num_kv_heads)
         scratch = self._make_scratch(bs, nsplit)
-        # warm up allocator/kernels on a side stream, then capture
+        # warm up allocator/kernels on a side stream, then capture.  The
+        # warm-up runs execute the step: K/V appends are idempotent, but a
+        # recurrent state would advance once per run, so stateful models warm
+        # up on the null slot and get their lanes' slots back afterwards
+        # (the graph holds the buffer, not its content).
+        real_slots = None
+        if self.stateful:
+            real_slots = self._dec["sslot"][:bs].clone()
+            self._dec["sslot"][:bs].zero_()
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
@@ -959,6 +967,8 @@ class LLMEngine:
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             self._decode_forward(bs, nsplit, scratch, tkp, lp)
+        if real_slots is not None:
+            self._dec["sslot"][:bs].copy_(real_slots)
         entry = {"graph": g, "nsplit": nsplit, "scratch": scratch}
         self._graphs[key] = entry
         return entry
