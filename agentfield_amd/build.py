@@ -48,7 +48,8 @@ HIP_SOURCES = [
 MIX_GROUPS = {
     "glue": (PKG_DIR / "libafglue.so", ["mix_glue.hip"]),
     "seq": (PKG_DIR / "libafmix.so", ["mix_seq.hip", "mix_attn_mfma.hip"]),
-    "ssm": (PKG_DIR / "libafssm.so", ["mix_ssm.hip", "mix_sigattn.hip"]),
+    "ssm": (PKG_DIR / "libafssm.so", ["mix_ssm.hip", "mix_sigattn.hip",
+                                       "mix_sigattn_mfma.hip"]),
 }
 MIX_SOURCES = [s for _lib, srcs in MIX_GROUPS.values() for s in srcs]
 MIX_LIB = MIX_GROUPS["seq"][0]

@@ -161,6 +161,9 @@ def _mix_sigs() -> dict:
                                    p, i, i, i, i, p],
             "afm_qk_unit_cache": [p, p, i64, p, i64, p, i64, p, i64, f, p, p,
                                   p, p, f, f, i, i, i, i, i, i, i, i, p],
+            "afm_sigattn_prefill_mfma": [p, p, p, p, p, p, p, p, p, p, p, i, i,
+                                         p, p, p, i64, f, i, i, i, i, i, i, i,
+                                         p],
             "afm_sigmoid_attention": [p, p, p, p, p, p, p, p, p, p, i, i, p, p,
                                       p, i64, f, i, i, i, i, i, i, i, i, i, i,
                                       p],

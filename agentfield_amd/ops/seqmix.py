@@ -832,6 +832,30 @@ def sigmoid_attention(q: torch.Tensor, kcache: torch.Tensor,
             out = out * torch.sigmoid(gate.float())[:, :, None]
         return out.view(T, H * dv).to(q.dtype)
     out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+    lens = getattr(md, "seq_lens", None)
+    if (q.dtype == torch.bfloat16 and lens is not None and window == 0
+            and dk <= 128 and dv <= 128 and H <= 16
+            and max(lens) >= MFMA_MIN_ROWS):
+        # prompt portions: 16-row tiles x all heads on the matrix cores
+        ts, tq = [], []
+        for b, ln in enumerate(lens):
+            for q0 in range(0, ln, 16):
+                ts.append(b)
+                tq.append(q0)
+        tile_seq = torch.tensor(ts, dtype=torch.int32, device=q.device)
+        tile_q0 = torch.tensor(tq, dtype=torch.int32, device=q.device)
+        rc = _L().afm_sigattn_prefill_mfma(
+            _lib.ptr(out), _lib.ptr(q), _lib.ptr(kcache), _lib.ptr(vcache),
+            _lib.ptr(md.block_table), _lib.ptr(md.cu_seqlens),
+            _lib.ptr(md.q_start), _lib.ptr(tile_seq), _lib.ptr(tile_q0),
+            _lib.ptr(rel), _lib.ptr(buckets),
+            buckets.numel() if buckets is not None else 0, RB,
+            _lib.ptr(talk), _lib.ptr(head_bias), _lib.ptr(gate),
+            _rowstride(gate) if gate is not None else 0, float(scale),
+            len(ts), H, G, dk, dv, page, md.block_table.shape[1],
+            _lib.cur_stream())
+        _lib.check(rc, "afm_sigattn_prefill_mfma")
+        return out
     # few rows and a long reach: cut each row's keys over several workgroups
     reach = md.block_table.shape[1] * page
     if window > 0:
