@@ -317,7 +317,7 @@ __global__ void __launch_bounds__(256) cast_rows_kernel(
 //   u = y (+ bias);  x += u / sqrt(mean(u^2) + eps) * w;  h = S(x)
 // y is [T, W] in Y (storage dtype or fp32), x the fp32 residual, h an
 // optional copy of the new residual row in the storage dtype.
-template <typename S, typename Y>
+template <typename S, typename Y, int V>
 __global__ void __launch_bounds__(256) norm_residual_kernel(
     float* __restrict__ x, S* __restrict__ h, const Y* __restrict__ y,
     i64 ldy, const S* __restrict__ bias, const S* __restrict__ w, float eps,
@@ -326,18 +326,26 @@ __global__ void __launch_bounds__(256) norm_residual_kernel(
   const int t = blockIdx.x;
   const Y* yr = y + (size_t)t * ldy;
   float ss[1] = {0.f};
-  for (int i = threadIdx.x; i < W; i += 256) {
-    const float u = ldf<Y>(yr + i) + (bias ? ldf<S>(bias + i) : 0.f);
-    ss[0] += u * u;
+  for (int i = threadIdx.x * V; i < W; i += 256 * V) {
+    float u[4], bv[4] = {0.f, 0.f, 0.f, 0.f};
+    ldv<Y, V>(yr + i, u);
+    if (bias) ldv<S, V>(bias + i, bv);
+#pragma unroll
+    for (int j = 0; j < V; ++j) { u[j] += bv[j]; ss[0] += u[j] * u[j]; }
   }
   block_sum<1>(ss, red);
   const float rs = 1.0f / sqrtf(ss[0] / (float)W + eps);
   float* xr = x + (size_t)t * W;
-  for (int i = threadIdx.x; i < W; i += 256) {
-    const float u = ldf<Y>(yr + i) + (bias ? ldf<S>(bias + i) : 0.f);
-    const float v = xr[i] + u * rs * ldf<S>(w + i);
-    xr[i] = v;
-    if (h) stf<S>(h + (size_t)t * W + i, v);
+  for (int i = threadIdx.x * V; i < W; i += 256 * V) {
+    float u[4], bv[4] = {0.f, 0.f, 0.f, 0.f}, wv[4], xv[4];
+    ldv<Y, V>(yr + i, u);
+    if (bias) ldv<S, V>(bias + i, bv);
+    ldv<S, V>(w + i, wv);
+    ldv<float, V>(xr + i, xv);
+#pragma unroll
+    for (int j = 0; j < V; ++j) xv[j] += (u[j] + bv[j]) * rs * wv[j];
+    stv<float, V>(xr + i, xv);
+    if (h) stv<S, V>(h + (size_t)t * W + i, xv);
   }
 }
 
@@ -347,27 +355,36 @@ __global__ void __launch_bounds__(256) norm_residual_kernel(
 // e.g. a router weight per (token, expert) row) are optional.  Row r sits at
 // (r / rg) * ld + (r % rg) * ld_in, so rg units laid side by side in one
 // matrix row (experts of one token) are rows of their own.
-template <typename S, int ACT>
+template <typename S, int ACT, int V>
 __global__ void __launch_bounds__(256) glu_kernel(
     S* __restrict__ out, i64 ldo, i64 ldo_in, const S* __restrict__ g,
     const S* __restrict__ u, i64 ldi, i64 ldi_in, int rg,
     const S* __restrict__ bg, const S* __restrict__ bu,
     const float* __restrict__ rw, i64 R, int F) {
-  const i64 n = R * F;
+  const int FV = F / V;
+  const i64 n = R * FV;
   for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n;
        i += (i64)gridDim.x * 256) {
-    const i64 r = i / F;
-    const int c = (int)(i % F);
+    const i64 r = i / FV;
+    const int c = (int)(i % FV) * V;
     const i64 ri = (r / rg) * ldi + (r % rg) * ldi_in;
-    float a = ldf<S>(g + ri + c) + (bg ? ldf<S>(bg + c) : 0.f);
-    const float b = ldf<S>(u + ri + c) + (bu ? ldf<S>(bu + c) : 0.f);
-    if (ACT == 0) a = a / (1.0f + expf(-a));
-    else if (ACT == 1) a = fmaxf(a, 0.f);
-    else a = 0.5f * a * (1.0f + tanhf(0.7978845608028654f *
-                                      (a + 0.044715f * a * a * a)));
-    float o = a * b;
-    if (rw) o *= rw[r];
-    stf<S>(out + (r / rg) * ldo + (r % rg) * ldo_in + c, o);
+    float a[4], b[4], ba[4] = {0.f, 0.f, 0.f, 0.f}, bb[4] = {0.f, 0.f, 0.f, 0.f};
+    ldv<S, V>(g + ri + c, a);
+    ldv<S, V>(u + ri + c, b);
+    if (bg) ldv<S, V>(bg + c, ba);
+    if (bu) ldv<S, V>(bu + c, bb);
+    const float wr = rw ? rw[r] : 1.0f;
+    float o[4];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      float av = a[j] + ba[j];
+      if (ACT == 0) av = av / (1.0f + expf(-av));
+      else if (ACT == 1) av = fmaxf(av, 0.f);
+      else av = 0.5f * av * (1.0f + tanhf(0.7978845608028654f *
+                                          (av + 0.044715f * av * av * av)));
+      o[j] = av * (b[j] + bb[j]) * wr;
+    }
+    stv<S, V>(out + (r / rg) * ldo + (r % rg) * ldo_in + c, o);
   }
 }
 
@@ -635,9 +652,16 @@ AF_EXPORT int afm_norm_residual(void* x, void* h, const void* y, i64 ldy,
                                 void* stream) {
   if (T == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  const bool vec = W % 4 == 0 && ldy % 4 == 0 && aligned16(x, h, y, bias, w);
 #define NR(ST, YT)                                                          \
-  norm_residual_kernel<ST, YT><<<T, 256, 0, s>>>((float*)x, (ST*)h,         \
-      (const YT*)y, ldy, (const ST*)bias, (const ST*)w, eps, W)
+  do {                                                                      \
+    if (vec)                                                                \
+      norm_residual_kernel<ST, YT, 4><<<T, 256, 0, s>>>((float*)x, (ST*)h,  \
+          (const YT*)y, ldy, (const ST*)bias, (const ST*)w, eps, W);        \
+    else                                                                    \
+      norm_residual_kernel<ST, YT, 1><<<T, 256, 0, s>>>((float*)x, (ST*)h,  \
+          (const YT*)y, ldy, (const ST*)bias, (const ST*)w, eps, W);        \
+  } while (0)
   if (dt == 0) { if (y_f32) NR(u16, float); else NR(u16, u16); }
   else if (dt == 1) NR(float, float);
   else return 9002;
@@ -652,11 +676,21 @@ AF_EXPORT int afm_glu(void* out, i64 ldo, i64 ldo_in, const void* g,
   if (R == 0 || F == 0) return 0;
   if (act < 0 || act > 2 || rg < 1) return 9003;
   hipStream_t s = (hipStream_t)stream;
-  const int grid = grid_for(R * F);
+  const bool vec = F % 4 == 0 && ldo % 4 == 0 && ldo_in % 4 == 0 &&
+                   ldi % 4 == 0 && ldi_in % 4 == 0 &&
+                   aligned16(out, g, u, bg, bu);
+  const int grid = grid_for(R * F / (vec ? 4 : 1));
 #define GLU(ST, A)                                                         \
-  glu_kernel<ST, A><<<grid, 256, 0, s>>>((ST*)out, ldo, ldo_in,            \
-      (const ST*)g, (const ST*)u, ldi, ldi_in, rg, (const ST*)bg,          \
-      (const ST*)bu, (const float*)rw, R, F)
+  do {                                                                     \
+    if (vec)                                                               \
+      glu_kernel<ST, A, 4><<<grid, 256, 0, s>>>((ST*)out, ldo, ldo_in,     \
+          (const ST*)g, (const ST*)u, ldi, ldi_in, rg, (const ST*)bg,      \
+          (const ST*)bu, (const float*)rw, R, F);                          \
+    else                                                                   \
+      glu_kernel<ST, A, 1><<<grid, 256, 0, s>>>((ST*)out, ldo, ldo_in,     \
+          (const ST*)g, (const ST*)u, ldi, ldi_in, rg, (const ST*)bg,      \
+          (const ST*)bu, (const float*)rw, R, F);                          \
+  } while (0)
 #define GLU_ACT(ST)                                   \
   do {                                                \
     if (act == 0) GLU(ST, 0);                         \

@@ -85,6 +85,73 @@ __global__ void __launch_bounds__(256) qk_unit_cache_kernel(
   }
 }
 
+// The same with 16-byte accesses: LPH = dk / EPL lanes share a head (a power
+// of two), a wave takes 64 / LPH heads per pass.
+template <typename S>
+__device__ __forceinline__ void st16(S* p, const float* o) {
+  if constexpr (sizeof(S) == 2) {
+    s16x8 v;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (short)f2bf(o[j]);
+    *reinterpret_cast<s16x8*>(p) = v;
+  } else {
+    *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+  }
+}
+
+template <typename S>
+__global__ void __launch_bounds__(256) qk_unit_cache_vec_kernel(
+    S* __restrict__ qout, const S* __restrict__ q, i64 ldq,
+    const S* __restrict__ k, i64 ldk, const S* __restrict__ v, i64 ldv,
+    const S* __restrict__ vfirst, i64 ldvf, float lam, S* __restrict__ kc,
+    S* __restrict__ vc, const i64* __restrict__ slots,
+    const i32* __restrict__ positions, float eps, float t_coef, int t_every,
+    int H, int G, int dk, int dv, int page, int lph) {
+  constexpr int EPL = Epl<S>::n;
+  const int t = blockIdx.x;
+  const i64 sl = slots[t];
+  const i64 pg = sl >= 0 ? sl / page : 0, off = sl >= 0 ? sl % page : 0;
+  float temp = 1.0f;
+  if (t_every > 0)
+    temp = 1.0f + t_coef * logf((float)((positions[t] + 1) / t_every) + 1.0f);
+  const int hpp = 256 / lph;                  // heads per pass
+  const int sub = threadIdx.x % lph;
+  for (int hh = threadIdx.x / lph; hh < H + G; hh += hpp) {
+    const bool isq = hh < H;
+    const S* src = (isq ? q + (size_t)t * ldq + (size_t)hh * dk
+                        : k + (size_t)t * ldk + (size_t)(hh - H) * dk) +
+                   sub * EPL;
+    float x[EPL];
+    ld16<S, true>(src, x);
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) ss += x[j] * x[j];
+    for (int o = lph >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    float r = 1.0f / sqrtf(ss / (float)dk + eps);
+    if (isq) r *= temp;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) x[j] *= r;
+    if (isq)
+      st16<S>(qout + ((size_t)t * H + hh) * dk + sub * EPL, x);
+    else if (sl >= 0)
+      st16<S>(kc + (((size_t)pg * G + (hh - H)) * page + off) * dk + sub * EPL,
+              x);
+  }
+  if (sl < 0) return;
+  for (int i = threadIdx.x * EPL; i < G * dv; i += 256 * EPL) {
+    const int g = i / dv, d = i % dv;
+    float x[EPL];
+    ld16<S, true>(v + (size_t)t * ldv + i, x);
+    if (vfirst) {
+      float f[EPL];
+      ld16<S, true>(vfirst + (size_t)t * ldvf + i, f);
+#pragma unroll
+      for (int j = 0; j < EPL; ++j) x[j] = (1.0f - lam) * x[j] + lam * f[j];
+    }
+    st16<S>(vc + (((size_t)pg * G + g) * page + off) * dv + d, x);
+  }
+}
+
 // --------------------------------------------------------------- attention
 // One workgroup per (row, key split).  Keys are walked in tiles of KT:
 //   A. one key per thread: its K rows are dotted with every head's query
@@ -96,7 +163,8 @@ __global__ void __launch_bounds__(256) qk_unit_cache_kernel(
 //   C. W.V: thread = (key group, 16-byte slice of one head's output); the
 //      key groups' partial sums are added through LDS at the end.
 // Partial outputs are fp32 [T, nsplit, H*dv].
-constexpr int ACCR = 4;   // output slices per thread when H*dv/EPL > 256
+// output slices per thread when H*dv/EPL > 256 (more in the scalar build)
+template <bool VEC> struct Accr { static constexpr int n = VEC ? 4 : 16; };
 
 template <typename S, int KT, bool VEC>
 __global__ void __launch_bounds__(256) sigmoid_attention_kernel(
@@ -109,6 +177,7 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(
     int H, int G, int dk, int dv, int page, int maxp, int nsplit,
     int window) {
   constexpr int EPL = VEC ? Epl<S>::n : 1;
+  constexpr int ACCR = Accr<VEC>::n;
   extern __shared__ float sh[];
   float* qs = sh;                         // [H*dk]
   float* sc = qs + H * dk;                // [H][KT]
@@ -130,8 +199,8 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(
 
   const int lo_all = window > 0 ? max(0, qi - window + 1) : 0;
   const int n_keys = qi + 1 - lo_all;
-  const int tiles = (n_keys + KT - 1) / KT;
-  const int per = (tiles + nsplit - 1) / nsplit * KT;
+  // even key ranges per split, in steps of 32 keys
+  const int per = ((n_keys + nsplit - 1) / nsplit + 31) / 32 * 32;
   const int lo = lo_all + split * per;
   const int hi = min(qi + 1, lo + per);
 
@@ -214,9 +283,28 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(
           const int h = (e * EPL) / dv, d = (e * EPL) % dv;
           const int g = h / rep;
           const float* wh = wt + h * KT;
-          for (int jj = kg; jj < cnt; jj += KG) {
+          const S* vbase = vc + (size_t)g * page * dv + d;
+          int jj = kg;
+          // four value rows in flight per thread
+          for (; jj + 3 * KG < cnt; jj += 4 * KG) {
+            float v0[EPL], v1[EPL], v2[EPL], v3[EPL];
+            ld16<S, VEC>(vbase + (size_t)koff[jj] * dv, v0);
+            ld16<S, VEC>(vbase + (size_t)koff[jj + KG] * dv, v1);
+            ld16<S, VEC>(vbase + (size_t)koff[jj + 2 * KG] * dv, v2);
+            ld16<S, VEC>(vbase + (size_t)koff[jj + 3 * KG] * dv, v3);
+            const float w0 = wh[jj], w1 = wh[jj + KG], w2 = wh[jj + 2 * KG],
+                        w3 = wh[jj + 3 * KG];
+#pragma unroll
+            for (int x = 0; x < EPL; ++x) {
+              acc[r][x] += w0 * v0[x];
+              acc[r][x] += w1 * v1[x];
+              acc[r][x] += w2 * v2[x];
+              acc[r][x] += w3 * v3[x];
+            }
+          }
+          for (; jj < cnt; jj += KG) {
             float vv[EPL];
-            ld16<S, VEC>(vc + (size_t)(koff[jj] + g * page) * dv + d, vv);
+            ld16<S, VEC>(vbase + (size_t)koff[jj] * dv, vv);
             const float w = wh[jj];
 #pragma unroll
             for (int x = 0; x < EPL; ++x) acc[r][x] += w * vv[x];
@@ -307,7 +395,8 @@ int dispatch_sig(float* part, const void* q, const void* kc, const void* vc,
   const bool vec = dk % EPLV == 0 && dv % EPLV == 0 &&
                    (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0;
   const int epl = vec ? EPLV : 1;
-  if ((i64)H * dv > (i64)256 * ACCR * epl) return 9004;
+  if ((i64)H * dv > (i64)256 * (vec ? Accr<true>::n : Accr<false>::n) * epl)
+    return 9004;
   auto lds = [&](int kt) {
     return ((size_t)H * dk + 2 * (size_t)H * kt + (size_t)H * H + H +
             (size_t)RB * H + kt + 256 * (size_t)epl) * sizeof(float);
@@ -342,11 +431,28 @@ AF_EXPORT int afm_qk_unit_cache(
   if (T == 0) return 0;
   if (H < 1 || G < 1 || H % G != 0) return 9003;
   hipStream_t s = (hipStream_t)stream;
+  auto al = [](const void* p) { return (uintptr_t)p % 16 == 0; };
 #define QKU(ST)                                                              \
-  qk_unit_cache_kernel<ST><<<T, 256, 0, s>>>((ST*)qout, (const ST*)q, ldq,   \
-      (const ST*)k, ldk, (const ST*)v, ldv, (const ST*)vfirst, ldvf, lam,    \
-      (ST*)kc, (ST*)vc, (const i64*)slots, (const i32*)positions, eps,       \
-      t_coef, t_every, H, G, dk, dv, page)
+  do {                                                                       \
+    constexpr int E = 16 / (int)sizeof(ST);                                  \
+    const int lph = dk / E;                                                  \
+    const bool vec = dk % E == 0 && dv % E == 0 && lph >= 1 && lph <= 64 && \
+                     (lph & (lph - 1)) == 0 && ldq % E == 0 &&               \
+                     ldk % E == 0 && ldv % E == 0 && ldvf % E == 0 &&        \
+                     al(qout) && al(q) && al(k) && al(v) && al(vfirst) &&    \
+                     al(kc) && al(vc);                                       \
+    if (vec)                                                                 \
+      qk_unit_cache_vec_kernel<ST><<<T, 256, 0, s>>>((ST*)qout,              \
+          (const ST*)q, ldq, (const ST*)k, ldk, (const ST*)v, ldv,           \
+          (const ST*)vfirst, ldvf, lam, (ST*)kc, (ST*)vc,                    \
+          (const i64*)slots, (const i32*)positions, eps, t_coef, t_every,    \
+          H, G, dk, dv, page, lph);                                          \
+    else                                                                     \
+      qk_unit_cache_kernel<ST><<<T, 256, 0, s>>>((ST*)qout, (const ST*)q,    \
+          ldq, (const ST*)k, ldk, (const ST*)v, ldv, (const ST*)vfirst,      \
+          ldvf, lam, (ST*)kc, (ST*)vc, (const i64*)slots,                    \
+          (const i32*)positions, eps, t_coef, t_every, H, G, dk, dv, page);  \
+  } while (0)
   if (dt == 0) QKU(u16);
   else if (dt == 1) QKU(float);
   else return 9002;

@@ -27,32 +27,67 @@ template <> __device__ __forceinline__ float decay_exp<float>(float v) { return 
 // before the chunk come from the sequence's slot of `state`
 // [slots, taps-1, C] (the taps-1 inputs before the chunk, oldest first),
 // inputs before position 0 are zero.  One thread per (row, channel).
-template <typename S>
+// V consecutive channels per thread (V = 4: 8- or 16-byte accesses).
+template <typename S, int V>
+__device__ __forceinline__ void ldc(const S* p, float (&o)[4]) {
+  if constexpr (V == 1) {
+    o[0] = ldf<S>(p);
+  } else if constexpr (sizeof(S) == 2) {
+    const s16x4 v = *reinterpret_cast<const s16x4*>(p);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = bf2f((u16)v[j]);
+  } else {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(p);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = v[j];
+  }
+}
+template <typename S, int V>
+__device__ __forceinline__ void stc(S* p, const float (&o)[4]) {
+  if constexpr (V == 1) {
+    stf<S>(p, o[0]);
+  } else if constexpr (sizeof(S) == 2) {
+    s16x4 v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = (short)f2bf(o[j]);
+    *reinterpret_cast<s16x4*>(p) = v;
+  } else {
+    *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+  }
+}
+
+template <typename S, int V>
 __global__ void __launch_bounds__(256) causal_conv_kernel(
     S* __restrict__ out, const S* __restrict__ in, i64 ldi,
     const S* __restrict__ w, const S* __restrict__ bias,
     const S* __restrict__ state, const i32* __restrict__ row_seq,
     const i32* __restrict__ cu, const i32* __restrict__ q_start,
     const i32* __restrict__ sslot, i64 n, int C, int taps, int silu) {
+  const int CV = C / V;
   for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n;
        i += (i64)gridDim.x * 256) {
-    const int t = (int)(i / C), c = (int)(i % C);
+    const int t = (int)(i / CV), c = (int)(i % CV) * V;
     const int b = row_seq[t];
     const int r0 = cu[b];
     const int k = t - r0;                 // row inside the chunk
     const int pos = q_start[b] + k;
     const S* st = state + (size_t)sslot[b] * (taps - 1) * C;
-    float acc = bias ? ldf<S>(bias + c) : 0.f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias) ldc<S, V>(bias + c, acc);
     for (int l = 0; l < taps; ++l) {      // lag
       if (pos - l < 0) break;
-      const float wv = ldf<S>(w + (size_t)c * taps + (taps - 1 - l));
-      float v;
-      if (l <= k) v = ldf<S>(in + (size_t)(t - l) * ldi + c);
-      else v = ldf<S>(st + (size_t)(taps - 1 - (l - k)) * C + c);
-      acc += wv * v;
+      float v[4];
+      if (l <= k) ldc<S, V>(in + (size_t)(t - l) * ldi + c, v);
+      else ldc<S, V>(st + (size_t)(taps - 1 - (l - k)) * C + c, v);
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        acc[j] += ldf<S>(w + (size_t)(c + j) * taps + (taps - 1 - l)) * v[j];
     }
-    if (silu) acc = acc / (1.0f + expf(-acc));
-    stf<S>(out + (size_t)t * C + c, acc);
+    if (silu) {
+#pragma unroll
+      for (int j = 0; j < V; ++j) acc[j] = acc[j] / (1.0f + expf(-acc[j]));
+    }
+    stc<S, V>(out + (size_t)t * C + c, acc);
   }
 }
 
@@ -85,17 +120,33 @@ __global__ void __launch_bounds__(256) conv_state_kernel(
 }
 
 // ---------------------------------------------------------- selective scan
-// Workgroup = (block of CB = 16 channels, sequence); 256 threads = 16
-// channels x 16 state lanes, lane l keeping states n = l, l+16, ... (PER of
-// them) of its channel in registers.  Tokens are staged TB at a time into
-// LDS (step size after softplus, input, silu(z), B and C rows), then walked serially:
+// Workgroup = (block of CB channels, sequence); 256 threads = CB channels x
+// NL state lanes (NL = 4, CB = 64 for N <= 64; NL = 16, CB = 16 beyond),
+// lane l keeping the PER consecutive states n = l*PER .. l*PER+PER-1 of its
+// channel in registers.  Tokens are staged TB at a time into LDS (step size
+// after softplus, input, silu(z), B and C rows), then walked serially:
 //   S[c,n] = exp(dt_c A[c,n]) S[c,n] + dt_c x_c B_n ;  y_c = sum_n S[c,n] C_n
-// with the sum over the 16 lanes taken by shuffles.  The output is
-// (y + D x) * silu(z) in the storage dtype.
-constexpr int SCAN_CB = 16;
+// with the sum over the NL lanes taken by DPP / shuffles.  The outputs of a
+// token block, (y + D x) * silu(z), leave through LDS as contiguous row
+// segments in the storage dtype.
 constexpr int SCAN_TB = 16;
 
-template <typename S, int PER>
+template <int NL>
+__device__ __forceinline__ float lanes_sum(float v) {
+  if constexpr (NL == 4) {
+    // quad_perm [1,0,3,2] and [2,3,0,1]: xor 1, xor 2 inside a quad
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+        0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+        0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));
+  } else {
+#pragma unroll
+    for (int o = NL / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  }
+  return v;
+}
+
+template <typename S, int NL, int PER>
 __global__ void __launch_bounds__(256) selective_scan_kernel(
     S* __restrict__ out, float* __restrict__ state, const S* __restrict__ x,
     const S* __restrict__ dtp, const S* __restrict__ dt_bias,
@@ -103,17 +154,19 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(
     const float* __restrict__ A, const float* __restrict__ D,
     const i32* __restrict__ cu, const i32* __restrict__ q_start,
     const i32* __restrict__ sslot, int C, int N) {
+  constexpr int CB = 256 / NL;
   extern __shared__ float sh[];
   float* s_dt = sh;                              // [TB][CB]
-  float* s_x = s_dt + SCAN_TB * SCAN_CB;         // [TB][CB]
-  float* s_b = s_x + SCAN_TB * SCAN_CB;          // [TB][N]
+  float* s_x = s_dt + SCAN_TB * CB;              // [TB][CB]
+  float* s_z = s_x + SCAN_TB * CB;               // [TB][CB], silu(z)
+  float* s_y = s_z + SCAN_TB * CB;               // [TB][CB]
+  float* s_b = s_y + SCAN_TB * CB;               // [TB][N]
   float* s_c = s_b + SCAN_TB * N;                // [TB][N]
-  float* s_z = s_c + SCAN_TB * N;                // [TB][CB], silu(z)
   const int b = blockIdx.y;
   const int r0 = cu[b], L = cu[b + 1] - r0;
   if (L == 0) return;
-  const int c0 = blockIdx.x * SCAN_CB;
-  const int cl = threadIdx.x >> 4, lane = threadIdx.x & 15;
+  const int c0 = blockIdx.x * CB;
+  const int cl = threadIdx.x / NL, lane = threadIdx.x % NL;
   const int c = c0 + cl;
   const bool okc = c < C;
   float* sb = state + ((size_t)sslot[b] * C + (okc ? c : 0)) * N;
@@ -121,7 +174,7 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(
   const bool fresh = q_start[b] == 0;
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
-    const int n = lane + 16 * j;
+    const int n = lane * PER + j;
     const bool ok = okc && n < N;
     st[j] = (ok && !fresh) ? sb[n] : 0.f;
     a[j] = ok ? A[(size_t)c * N + n] : 0.f;
@@ -130,49 +183,52 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(
   for (int tb = 0; tb < L; tb += SCAN_TB) {
     const int nt = min(SCAN_TB, L - tb);
     __syncthreads();                   // previous block fully consumed
-    {
-      const int tt = threadIdx.x >> 4, cc = threadIdx.x & 15;   // [TB][CB]
-      if (tt < nt && c0 + cc < C) {
+    for (int i = threadIdx.x; i < nt * CB; i += 256) {
+      const int tt = i / CB, cc = i % CB;
+      if (c0 + cc < C) {
         const size_t row = (size_t)(r0 + tb + tt);
         const float v = ldf<S>(dtp + row * C + c0 + cc) +
                         ldf<S>(dt_bias + c0 + cc);
-        s_dt[tt * SCAN_CB + cc] = v > 20.f ? v : log1pf(expf(v));
-        s_x[tt * SCAN_CB + cc] = ldf<S>(x + row * C + c0 + cc);
+        s_dt[i] = v > 20.f ? v : log1pf(expf(v));
+        s_x[i] = ldf<S>(x + row * C + c0 + cc);
         const float zv = ldf<S>(z + row * ldz + c0 + cc);
-        s_z[tt * SCAN_CB + cc] = zv / (1.0f + expf(-zv));
+        s_z[i] = zv / (1.0f + expf(-zv));
       }
-      for (int i = threadIdx.x; i < nt * N; i += 256) {
-        const int t2 = i / N, n = i % N;
-        const S* rowp = bc + (size_t)(r0 + tb + t2) * ldbc;
-        s_b[t2 * N + n] = ldf<S>(rowp + n);
-        s_c[t2 * N + n] = ldf<S>(rowp + N + n);
-      }
+    }
+    for (int i = threadIdx.x; i < nt * N; i += 256) {
+      const int t2 = i / N, n = i % N;
+      const S* rowp = bc + (size_t)(r0 + tb + t2) * ldbc;
+      s_b[i] = ldf<S>(rowp + n);
+      s_c[i] = ldf<S>(rowp + N + n);
     }
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
-      const float dt = s_dt[tt * SCAN_CB + cl];
-      const float xv = s_x[tt * SCAN_CB + cl];
+      const float dt = s_dt[tt * CB + cl];
+      const float xv = s_x[tt * CB + cl];
       const float dx = dt * xv;
       float y = 0.f;
 #pragma unroll
       for (int j = 0; j < PER; ++j) {
-        const int n = lane + 16 * j;
+        const int n = lane * PER + j;
         if (n < N) {
           st[j] = decay_exp<S>(dt * a[j]) * st[j] + dx * s_b[tt * N + n];
           y += st[j] * s_c[tt * N + n];
         }
       }
-#pragma unroll
-      for (int o = 8; o > 0; o >>= 1) y += __shfl_xor(y, o, 64);
-      if (lane == 0 && okc) {
-        stf<S>(out + (size_t)(r0 + tb + tt) * C + c,
-               (y + dcoef * xv) * s_z[tt * SCAN_CB + cl]);
-      }
+      y = lanes_sum<NL>(y);
+      if (lane == 0)
+        s_y[tt * CB + cl] = (y + dcoef * xv) * s_z[tt * CB + cl];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nt * CB; i += 256) {
+      const int tt = i / CB, cc = i % CB;
+      if (c0 + cc < C)
+        stf<S>(out + (size_t)(r0 + tb + tt) * C + c0 + cc, s_y[i]);
     }
   }
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
-    const int n = lane + 16 * j;
+    const int n = lane * PER + j;
     if (okc && n < N) sb[n] = st[j];
   }
 }
@@ -193,13 +249,18 @@ AF_EXPORT int afm_causal_conv(void* out, const void* in, i64 ldi,
   if (T == 0) return 0;
   if (taps < 1 || (taps > 1 && !state)) return 9003;
   hipStream_t s = (hipStream_t)stream;
-  const i64 n = (i64)T * C;
+  const bool vec = C % 4 == 0 && ldi % 4 == 0 && (uintptr_t)out % 16 == 0 &&
+                   (uintptr_t)in % 16 == 0 && (uintptr_t)bias % 16 == 0 &&
+                   (uintptr_t)state % 16 == 0;
+  const i64 n = (i64)T * C / (vec ? 4 : 1);
+#define CONVK(ST, V)                                                         \
+  causal_conv_kernel<ST, V><<<grid_for(n), 256, 0, s>>>((ST*)out,            \
+      (const ST*)in, ldi, (const ST*)w, (const ST*)bias, (const ST*)state,   \
+      (const i32*)row_seq, (const i32*)cu, (const i32*)q_start,              \
+      (const i32*)sslot, n, C, taps, silu)
 #define CONV(ST)                                                             \
   do {                                                                       \
-    causal_conv_kernel<ST><<<grid_for(n), 256, 0, s>>>((ST*)out,             \
-        (const ST*)in, ldi, (const ST*)w, (const ST*)bias, (const ST*)state, \
-        (const i32*)row_seq, (const i32*)cu, (const i32*)q_start,            \
-        (const i32*)sslot, n, C, taps, silu);                                \
+    if (vec) CONVK(ST, 4); else CONVK(ST, 1);                                \
     if (taps > 1)                                                            \
       conv_state_kernel<ST><<<grid_for((i64)B * C), 256, 0, s>>>(            \
           (ST*)state, (const ST*)in, ldi, (const i32*)cu,                    \
@@ -208,6 +269,7 @@ AF_EXPORT int afm_causal_conv(void* out, const void* in, i64 ldi,
   if (dt == 0) CONV(u16);
   else if (dt == 1) CONV(float);
   else return 9002;
+#undef CONVK
 #undef CONV
   return af_last_err();
 }
@@ -222,21 +284,29 @@ AF_EXPORT int afm_selective_scan(void* out, void* state, const void* x,
   if (B == 0) return 0;
   if (N < 1 || N > 256) return 9003;
   hipStream_t s = (hipStream_t)stream;
-  const size_t sm = (size_t)SCAN_TB * (3 * SCAN_CB + 2 * N) * sizeof(float);
-  dim3 grid((C + SCAN_CB - 1) / SCAN_CB, B);
-  const int per = (N + 15) / 16;
-#define SCAN(ST, P)                                                           \
-  selective_scan_kernel<ST, P><<<grid, 256, sm, s>>>((ST*)out, (float*)state, \
-      (const ST*)x, (const ST*)dtp, (const ST*)dt_bias, (const ST*)bc, ldbc,  \
-      (const ST*)z, ldz, (const float*)A, (const float*)D, (const i32*)cu,    \
-      (const i32*)q_start, (const i32*)sslot, C, N)
-#define SCAN_PER(ST)                          \
-  do {                                        \
-    if (per <= 1) SCAN(ST, 1);                \
-    else if (per <= 2) SCAN(ST, 2);           \
-    else if (per <= 4) SCAN(ST, 4);           \
-    else if (per <= 8) SCAN(ST, 8);           \
-    else SCAN(ST, 16);                        \
+  const int nl = N <= 64 ? 4 : 16;
+  const int cb = 256 / nl;
+  const size_t sm = (size_t)SCAN_TB * (4 * cb + 2 * N) * sizeof(float);
+  dim3 grid((C + cb - 1) / cb, B);
+  const int per = (N + nl - 1) / nl;
+#define SCAN(ST, NL, P)                                                       \
+  selective_scan_kernel<ST, NL, P><<<grid, 256, sm, s>>>((ST*)out,            \
+      (float*)state, (const ST*)x, (const ST*)dtp, (const ST*)dt_bias,        \
+      (const ST*)bc, ldbc, (const ST*)z, ldz, (const float*)A,                \
+      (const float*)D, (const i32*)cu, (const i32*)q_start,                   \
+      (const i32*)sslot, C, N)
+#define SCAN_PER(ST)                                \
+  do {                                              \
+    if (nl == 4) {                                  \
+      if (per <= 1) SCAN(ST, 4, 1);                 \
+      else if (per <= 2) SCAN(ST, 4, 2);            \
+      else if (per <= 4) SCAN(ST, 4, 4);            \
+      else if (per <= 8) SCAN(ST, 4, 8);            \
+      else SCAN(ST, 4, 16);                         \
+    } else {                                        \
+      if (per <= 8) SCAN(ST, 16, 8);                \
+      else SCAN(ST, 16, 16);                        \
+    }                                               \
   } while (0)
   if (dt == 0) SCAN_PER(u16);
   else if (dt == 1) SCAN_PER(float);

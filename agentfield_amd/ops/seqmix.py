@@ -860,7 +860,7 @@ def sigmoid_attention(q: torch.Tensor, kcache: torch.Tensor,
     reach = md.block_table.shape[1] * page
     if window > 0:
         reach = min(reach, window)
-    nsplit = max(1, min(16, 1024 // max(1, T), reach // 256))
+    nsplit = max(1, min(32, 2048 // max(1, T), reach // 64))
     part = torch.empty(T, nsplit, H * dv, dtype=torch.float32,
                        device=q.device)
     rc = _L().afm_sigmoid_attention(
