@@ -215,22 +215,30 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(
     for (int e = 0; e < EPL; ++e) acc[r][e] = 0.f;
   const i32* btr = bt + (size_t)seq * maxp;
 
-  for (int j0 = lo; j0 < hi; j0 += KT) {
-    const int cnt = min(KT, hi - j0);
+  // tile width actually walked: the split's keys, 32 .. KT (a power of two)
+  int ktw = 32;
+  while (ktw < KT && ktw < hi - lo) ktw <<= 1;
+  const int ngs = 256 / ktw;
+
+  for (int j0 = lo; j0 < hi; j0 += ktw) {
+    const int cnt = min(ktw, hi - j0);
     __syncthreads();            // previous tile's wt/koff consumed; qs ready
-    if (tid < KT) {
-      const int j = j0 + tid;
-      const bool valid = tid < cnt;
-      if (valid) {
+    {
+      // thread = (key kk, group slice gs): with a narrow tile the K/V groups
+      // of one key are dotted by 256 / KT threads side by side
+      const int NGS = ngs;
+      const int kk = tid % ktw, gs = tid / ktw;
+      const int j = j0 + kk;
+      if (kk < cnt) {
         const int pg = btr[j / page], off = j % page;
         const int base = pg * G * page + off;
-        koff[tid] = base;
+        if (gs == 0) koff[kk] = base;
         int bk = 0;
         if (RB > 0) {
           const int n = qi - j;
           bk = n < n_tab ? bucket_tab[n] : RB - 1;
         }
-        for (int g = 0; g < G; ++g) {
+        for (int g = gs; g < G; g += NGS) {
           const S* kp = kc + (size_t)(base + g * page) * dk;
           for (int r0 = 0; r0 < rep; r0 += 8) {
             float a8[8];
@@ -252,26 +260,28 @@ __global__ void __launch_bounds__(256) sigmoid_attention_kernel(
             for (int r = 0; r < 8; ++r) {
               if (r0 + r < rep) {
                 const int h = g * rep + r0 + r;
-                sc[h * KT + tid] =
+                sc[h * KT + kk] =
                     a8[r] * scale + (RB > 0 ? rel_s[bk * H + h] : 0.f);
               }
             }
           }
         }
       }
-      for (int h = 0; h < H; ++h) {
+      if (NGS > 1) __syncthreads();   // a key's scores come from NGS threads
+      // the mix: thread = (key kk, heads gs, gs + NGS, ...)
+      for (int h = gs; h < H; h += NGS) {
         float w = 0.f;
-        if (valid) {
+        if (kk < cnt) {
           float m = pb_s[h];
           if (talk) {
             for (int g2 = 0; g2 < H; ++g2)
-              m += talk_s[h * H + g2] * sc[g2 * KT + tid];
+              m += talk_s[h * H + g2] * sc[g2 * KT + kk];
           } else {
-            m += sc[h * KT + tid];
+            m += sc[h * KT + kk];
           }
           w = 1.0f / (1.0f + expf(-m));
         }
-        wt[h * KT + tid] = w;
+        wt[h * KT + kk] = w;
       }
     }
     __syncthreads();
@@ -402,7 +412,7 @@ int dispatch_sig(float* part, const void* q, const void* kc, const void* vc,
             (size_t)RB * H + kt + 256 * (size_t)epl) * sizeof(float);
   };
   int kt = 256;
-  while (kt > 64 && lds(kt) > 64 * 1024) kt >>= 1;
+  while (kt > 32 && lds(kt) > 64 * 1024) kt >>= 1;
   const size_t sm = lds(kt);
   if (sm > 160 * 1024) return 9004;
 #define SIG(KT, V)                                                            \
@@ -412,11 +422,13 @@ int dispatch_sig(float* part, const void* q, const void* kc, const void* vc,
   if (vec) {
     if (kt == 256) SIG(256, true);
     if (kt == 128) SIG(128, true);
-    SIG(64, true);
+    if (kt == 64) SIG(64, true);
+    SIG(32, true);
   }
   if (kt == 256) SIG(256, false);
   if (kt == 128) SIG(128, false);
-  SIG(64, false);
+  if (kt == 64) SIG(64, false);
+  SIG(32, false);
 #undef SIG
 }
 

@@ -6,6 +6,7 @@
 // (exp), the state and its update are fp32; the scan walks tokens strictly
 // in order, so results do not depend on where a sequence was cut.
 #include "common.h"
+#include <stdlib.h>
 
 namespace {
 
@@ -21,12 +22,31 @@ template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p =
 template <typename S> __device__ __forceinline__ float decay_exp(float v);
 template <> __device__ __forceinline__ float decay_exp<u16>(float v) { return __expf(v); }
 template <> __device__ __forceinline__ float decay_exp<float>(float v) { return expf(v); }
+// softplus and silu of staged values, same split: hardware exp / log / rcp
+// behind bf16 inputs, library forms for fp32 storage
+template <typename S> __device__ __forceinline__ float softplus_f(float v);
+template <> __device__ __forceinline__ float softplus_f<u16>(float v) {
+  // far below zero log(1 + e^v) = e^v to rounding; 1 + e^v would lose it
+  return v > 20.f ? v : (v < -8.f ? __expf(v) : __logf(1.0f + __expf(v)));
+}
+template <> __device__ __forceinline__ float softplus_f<float>(float v) {
+  return v > 20.f ? v : log1pf(expf(v));
+}
+template <typename S> __device__ __forceinline__ float silu_f(float v);
+template <> __device__ __forceinline__ float silu_f<u16>(float v) {
+  return v * __frcp_rn(1.0f + __expf(-v));
+}
+template <> __device__ __forceinline__ float silu_f<float>(float v) {
+  return v / (1.0f + expf(-v));
+}
 
 // ------------------------------------------------------------- convolution
-// out[t, c] = silu(b[c] + sum_j w[c, j] * in[t - (taps-1-j), c]).  Inputs
+// out[t, c] = silu(b[c] + sum_j w[j, c] * in[t - (taps-1-j), c]), weights
+// tap-major [taps, C] so that neighbouring channels load together.  Inputs
 // before the chunk come from the sequence's slot of `state`
 // [slots, taps-1, C] (the taps-1 inputs before the chunk, oldest first),
-// inputs before position 0 are zero.  One thread per (row, channel).
+// inputs before position 0 are zero.  One workgroup per (row, 256*V
+// channels), V channels per thread.
 // V consecutive channels per thread (V = 4: 8- or 16-byte accesses).
 template <typename S, int V>
 __device__ __forceinline__ void ldc(const S* p, float (&o)[4]) {
@@ -62,33 +82,30 @@ __global__ void __launch_bounds__(256) causal_conv_kernel(
     const S* __restrict__ w, const S* __restrict__ bias,
     const S* __restrict__ state, const i32* __restrict__ row_seq,
     const i32* __restrict__ cu, const i32* __restrict__ q_start,
-    const i32* __restrict__ sslot, i64 n, int C, int taps, int silu) {
-  const int CV = C / V;
-  for (i64 i = (i64)blockIdx.x * 256 + threadIdx.x; i < n;
-       i += (i64)gridDim.x * 256) {
-    const int t = (int)(i / CV), c = (int)(i % CV) * V;
-    const int b = row_seq[t];
-    const int r0 = cu[b];
-    const int k = t - r0;                 // row inside the chunk
-    const int pos = q_start[b] + k;
-    const S* st = state + (size_t)sslot[b] * (taps - 1) * C;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    if (bias) ldc<S, V>(bias + c, acc);
-    for (int l = 0; l < taps; ++l) {      // lag
-      if (pos - l < 0) break;
-      float v[4];
-      if (l <= k) ldc<S, V>(in + (size_t)(t - l) * ldi + c, v);
-      else ldc<S, V>(st + (size_t)(taps - 1 - (l - k)) * C + c, v);
+    const i32* __restrict__ sslot, int C, int taps, int silu) {
+  const int t = blockIdx.x;
+  const int c = (blockIdx.y * 256 + threadIdx.x) * V;
+  if (c >= C) return;
+  const int b = row_seq[t];
+  const int k = t - cu[b];                // row inside the chunk
+  const int pos = q_start[b] + k;
+  const S* st = state + (size_t)sslot[b] * (taps - 1) * C;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if (bias) ldc<S, V>(bias + c, acc);
+  for (int l = 0; l < taps; ++l) {        // lag
+    if (pos - l < 0) break;
+    float v[4], wv[4];
+    if (l <= k) ldc<S, V>(in + (size_t)(t - l) * ldi + c, v);
+    else ldc<S, V>(st + (size_t)(taps - 1 - (l - k)) * C + c, v);
+    ldc<S, V>(w + (size_t)(taps - 1 - l) * C + c, wv);
 #pragma unroll
-      for (int j = 0; j < V; ++j)
-        acc[j] += ldf<S>(w + (size_t)(c + j) * taps + (taps - 1 - l)) * v[j];
-    }
-    if (silu) {
-#pragma unroll
-      for (int j = 0; j < V; ++j) acc[j] = acc[j] / (1.0f + expf(-acc[j]));
-    }
-    stc<S, V>(out + (size_t)t * C + c, acc);
+    for (int j = 0; j < V; ++j) acc[j] += wv[j] * v[j];
   }
+  if (silu) {
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = silu_f<S>(acc[j]);
+  }
+  stc<S, V>(out + (size_t)t * C + c, acc);
 }
 
 // After the chunk: the slot keeps the last taps-1 inputs of the sequence.
@@ -121,7 +138,8 @@ __global__ void __launch_bounds__(256) conv_state_kernel(
 
 // ---------------------------------------------------------- selective scan
 // Workgroup = (block of CB channels, sequence); 256 threads = CB channels x
-// NL state lanes (NL = 4, CB = 64 for N <= 64; NL = 16, CB = 16 beyond),
+// NL state lanes (NL = 4, CB = 64, or NL = 16, CB = 16 for large N or few
+// sequences),
 // lane l keeping the PER consecutive states n = l*PER .. l*PER+PER-1 of its
 // channel in registers.  Tokens are staged TB at a time into LDS (step size
 // after softplus, input, silu(z), B and C rows), then walked serially:
@@ -133,16 +151,13 @@ constexpr int SCAN_TB = 16;
 
 template <int NL>
 __device__ __forceinline__ float lanes_sum(float v) {
-  if constexpr (NL == 4) {
-    // quad_perm [1,0,3,2] and [2,3,0,1]: xor 1, xor 2 inside a quad
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
-        0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
-        0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));
-  } else {
 #pragma unroll
-    for (int o = NL / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  }
+  for (int o = NL / 2; o >= 4; o >>= 1) v += __shfl_xor(v, o, 64);
+  // quad_perm [2,3,0,1] and [1,0,3,2]: xor 2, xor 1 inside a quad
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
   return v;
 }
 
@@ -189,10 +204,10 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(
         const size_t row = (size_t)(r0 + tb + tt);
         const float v = ldf<S>(dtp + row * C + c0 + cc) +
                         ldf<S>(dt_bias + c0 + cc);
-        s_dt[i] = v > 20.f ? v : log1pf(expf(v));
+        s_dt[i] = softplus_f<S>(v);
         s_x[i] = ldf<S>(x + row * C + c0 + cc);
         const float zv = ldf<S>(z + row * ldz + c0 + cc);
-        s_z[i] = zv / (1.0f + expf(-zv));
+        s_z[i] = silu_f<S>(zv);
       }
     }
     for (int i = threadIdx.x; i < nt * N; i += 256) {
@@ -202,7 +217,7 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(
       s_c[i] = ldf<S>(rowp + N + n);
     }
     __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
+    auto step = [&](int tt) {
       const float dt = s_dt[tt * CB + cl];
       const float xv = s_x[tt * CB + cl];
       const float dx = dt * xv;
@@ -218,7 +233,8 @@ __global__ void __launch_bounds__(256) selective_scan_kernel(
       y = lanes_sum<NL>(y);
       if (lane == 0)
         s_y[tt * CB + cl] = (y + dcoef * xv) * s_z[tt * CB + cl];
-    }
+    };
+    for (int tt = 0; tt < nt; ++tt) step(tt);
     __syncthreads();
     for (int i = threadIdx.x; i < nt * CB; i += 256) {
       const int tt = i / CB, cc = i % CB;
@@ -251,13 +267,15 @@ AF_EXPORT int afm_causal_conv(void* out, const void* in, i64 ldi,
   hipStream_t s = (hipStream_t)stream;
   const bool vec = C % 4 == 0 && ldi % 4 == 0 && (uintptr_t)out % 16 == 0 &&
                    (uintptr_t)in % 16 == 0 && (uintptr_t)bias % 16 == 0 &&
+                   (uintptr_t)w % 16 == 0 &&
                    (uintptr_t)state % 16 == 0;
-  const i64 n = (i64)T * C / (vec ? 4 : 1);
+  const int vw = vec ? 4 : 1;
+  dim3 grid(T, (C / vw + 255) / 256);
 #define CONVK(ST, V)                                                         \
-  causal_conv_kernel<ST, V><<<grid_for(n), 256, 0, s>>>((ST*)out,            \
+  causal_conv_kernel<ST, V><<<grid, 256, 0, s>>>((ST*)out,                   \
       (const ST*)in, ldi, (const ST*)w, (const ST*)bias, (const ST*)state,   \
       (const i32*)row_seq, (const i32*)cu, (const i32*)q_start,              \
-      (const i32*)sslot, n, C, taps, silu)
+      (const i32*)sslot, C, taps, silu)
 #define CONV(ST)                                                             \
   do {                                                                       \
     if (vec) CONVK(ST, 4); else CONVK(ST, 1);                                \
@@ -284,7 +302,14 @@ AF_EXPORT int afm_selective_scan(void* out, void* state, const void* x,
   if (B == 0) return 0;
   if (N < 1 || N > 256) return 9003;
   hipStream_t s = (hipStream_t)stream;
-  const int nl = N <= 64 ? 4 : 16;
+  // 4 state lanes per channel (64 channels per workgroup) when that still
+  // gives the chip enough workgroups, else 16 lanes (16 channels)
+  // (AFM_SCAN_MIN_WGS moves the switch-over, for tuning)
+  static const long min_wgs = [] {
+    const char* e = getenv("AFM_SCAN_MIN_WGS");
+    return e ? atol(e) : 1024L;
+  }();
+  const int nl = (N <= 64 && (i64)B * ((C + 63) / 64) >= min_wgs) ? 4 : 16;
   const int cb = 256 / nl;
   const size_t sm = (size_t)SCAN_TB * (4 * cb + 2 * N) * sizeof(float);
   dim3 grid((C + cb - 1) / cb, B);
@@ -295,23 +320,24 @@ AF_EXPORT int afm_selective_scan(void* out, void* state, const void* x,
       (const ST*)bc, ldbc, (const ST*)z, ldz, (const float*)A,                \
       (const float*)D, (const i32*)cu, (const i32*)q_start,                   \
       (const i32*)sslot, C, N)
+#define SCAN_NL(ST, NL)                             \
+  do {                                              \
+    if (per <= 1) SCAN(ST, NL, 1);                  \
+    else if (per <= 2) SCAN(ST, NL, 2);             \
+    else if (per <= 4) SCAN(ST, NL, 4);             \
+    else if (per <= 8) SCAN(ST, NL, 8);             \
+    else SCAN(ST, NL, 16);                          \
+  } while (0)
 #define SCAN_PER(ST)                                \
   do {                                              \
-    if (nl == 4) {                                  \
-      if (per <= 1) SCAN(ST, 4, 1);                 \
-      else if (per <= 2) SCAN(ST, 4, 2);            \
-      else if (per <= 4) SCAN(ST, 4, 4);            \
-      else if (per <= 8) SCAN(ST, 4, 8);            \
-      else SCAN(ST, 4, 16);                         \
-    } else {                                        \
-      if (per <= 8) SCAN(ST, 16, 8);                \
-      else SCAN(ST, 16, 16);                        \
-    }                                               \
+    if (nl == 4) SCAN_NL(ST, 4);                    \
+    else SCAN_NL(ST, 16);                           \
   } while (0)
   if (dt == 0) SCAN_PER(u16);
   else if (dt == 1) SCAN_PER(float);
   else return 9002;
 #undef SCAN_PER
+#undef SCAN_NL
 #undef SCAN
   return af_last_err();
 }

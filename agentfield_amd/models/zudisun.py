@@ -222,7 +222,7 @@ class SelectiveSSM(nn.Module):
         super().__init__()
         s = self.spec = spec
         self.w_in = nn.Parameter(torch.empty(2 * s.inner, width))
-        self.conv = nn.Parameter(torch.empty(s.inner, s.conv))
+        self.conv = nn.Parameter(torch.empty(s.conv, s.inner))  # tap-major
         self.conv_b = nn.Parameter(torch.empty(s.inner))
         self.w_x = nn.Parameter(torch.empty(s.dt_rank + 2 * s.state, s.inner))
         self.w_dt = nn.Parameter(torch.empty(s.inner, s.dt_rank))
@@ -479,7 +479,7 @@ class ZudisunForCausalLM(nn.Module):
             m = L.mixer
             if isinstance(m, SelectiveSSM):
                 put(m.w_in, get(mp + "in"))
-                put(m.conv, get(mp + "conv"))
+                put(m.conv, get(mp + "conv").t().contiguous())
                 put(m.conv_b, get(mp + "conv.b"))
                 put(m.w_x, get(mp + "x"))
                 put(m.w_dt, get(mp + "dt"))
@@ -561,7 +561,7 @@ class ZudisunForCausalLM(nn.Module):
             elif leaf == "embed":
                 rnd(p, 1.0)
             elif leaf == "conv":
-                rnd(p, p.shape[1] ** -0.5)
+                rnd(p, p.shape[0] ** -0.5)
             else:
                 rnd(p, p.shape[1] ** -0.5)
         for L in self.layers:

@@ -627,13 +627,13 @@ def moe_combine(ys: torch.Tensor, pos: torch.Tensor, weights: torch.Tensor,
 def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None,
                 state: torch.Tensor, md, silu: bool = True) -> torch.Tensor:
     """Depthwise causal convolution over packed chunks: out[t, c] = act(b[c]
-    + sum_j w[c, j] x[t - (taps-1-j), c]), the last column weighing the
-    current token.  Inputs from before a chunk come from the sequence's slot
+    + sum_j w[j, c] x[t - (taps-1-j), c]); w is tap-major [taps, C], its last
+    row weighing the current token.  Inputs from before a chunk come from the sequence's slot
     of `state` [slots, taps-1, C] (storage dtype, oldest first), inputs
     before position 0 are zero; afterwards the slot holds the sequence's last
     taps-1 inputs.  x [T, C] may be a strided view."""
     T, C = x.shape
-    taps = w.shape[1]
+    taps = w.shape[0]
     B = md.q_start.numel()
     if not _gpu(x):
         out = torch.empty(T, C, dtype=torch.float32)
@@ -651,7 +651,7 @@ def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None,
             if bias is not None:
                 acc += bias.float()
             for j in range(taps):
-                acc += wf[:, j] * cat[j:j + r1 - r0]
+                acc += wf[j] * cat[j:j + r1 - r0]
             out[r0:r1] = acc
             if taps > 1:
                 state[sl[b]][:taps - 1] = cat[-(taps - 1):].to(state.dtype)

@@ -232,7 +232,9 @@ def test_selective_ssm_alone(device, dtype, shape):
     for name, src in (("w_in", "in"), ("conv", "conv"), ("conv_b", "conv.b"),
                       ("w_x", "x"), ("w_dt", "dt"), ("dt_b", "dt.b"),
                       ("o", "o")):
-        getattr(mod, name).data = P["l0.mix." + src].clone()
+        w = P["l0.mix." + src]
+        getattr(mod, name).data = (w.t().contiguous() if name == "conv"
+                                   else w.clone())
     mod.A.copy_(-torch.exp(P["l0.mix.A_log"].float()))
     mod.D.copy_(P["l0.mix.D"].float())
     mod = mod.to(device)
@@ -262,7 +264,8 @@ def test_conv_history_shorter_than_taps(device):
     got, lo = [], 0
     for n in (1, 2, 1, 1, 3, 2, 7):
         md, _ = md_for([n], [lo], [1], device)
-        got.append(sm.causal_conv(x[lo:lo + n].to(device), w.to(device),
+        got.append(sm.causal_conv(x[lo:lo + n].to(device),
+                                  w.t().contiguous().to(device),
                                   b.to(device), state, md).cpu())
         lo += n
     assert torch.allclose(torch.cat(got).to(F64), want, atol=1e-5)
