@@ -6,7 +6,7 @@
 // The head mix needs the scores of ALL heads for a (row, key) pair before
 // any weight is known, and the output accumulators of all heads for a row
 // tile must stay on chip over the whole key walk.  So a workgroup takes 16
-// consecutive rows of one sequence and all heads; wave w owns HPW
+// consecutive rows of one sequence and all heads; wave w (of up to 8) owns HPW
 // consecutive heads (scores, weights and outputs of those heads).  Per tile
 // of 32 keys:
 //   1. every wave stages V of its K/V groups transposed into a private LDS
@@ -55,7 +55,7 @@ constexpr int KT = 32;    // keys per tile
 constexpr int VS = 40;    // LDS row stride of V^T / W tiles (32 keys + pad)
 
 template <int DKC, int DVT, int HPW, bool VEC>
-__global__ void __launch_bounds__(256) sigattn_prefill_mfma_kernel(
+__global__ void __launch_bounds__(512) sigattn_prefill_mfma_kernel(
     u16* __restrict__ out, const u16* __restrict__ q,
     const u16* __restrict__ kc, const u16* __restrict__ vc,
     const i32* __restrict__ bt, const i32* __restrict__ cu,
@@ -69,8 +69,9 @@ __global__ void __launch_bounds__(256) sigattn_prefill_mfma_kernel(
   f32x4* s_x = reinterpret_cast<f32x4*>(smem);            // [H][2][64]
   u16* v_all = reinterpret_cast<u16*>(s_x + (size_t)H * 2 * 64);
   const int vwave = ngw * DVT * 16 * VS;                  // elements per wave
-  u16* p_all = v_all + 4 * vwave;                         // [4][16][VS]
-  float* rel_s = reinterpret_cast<float*>(p_all + 4 * 16 * VS);   // [RB*H]
+  const int nwv = blockDim.x >> 6;                        // waves: 1..8
+  u16* p_all = v_all + nwv * vwave;                       // [nwv][16][VS]
+  float* rel_s = reinterpret_cast<float*>(p_all + nwv * 16 * VS);  // [RB*H]
   i32* tab_s = reinterpret_cast<i32*>(rel_s + RB * H);            // [n_tab]
 
   const int tile = blockIdx.x;
@@ -89,8 +90,9 @@ __global__ void __launch_bounds__(256) sigattn_prefill_mfma_kernel(
   const int nh = max(0, min(HPW, H - h0));  // and how many it has
   const int g0 = min(h0, H - 1) / rep;      // first K/V group it touches
 
-  for (int i = threadIdx.x; i < RB * H; i += 256) rel_s[i] = rel[i];
-  for (int i = threadIdx.x; i < n_tab; i += 256) tab_s[i] = bucket_tab[i];
+  for (int i = threadIdx.x; i < RB * H; i += blockDim.x) rel_s[i] = rel[i];
+  for (int i = threadIdx.x; i < n_tab; i += blockDim.x)
+    tab_s[i] = bucket_tab[i];
 
   s16x8 q_frag[HPW][DKC];
   {
@@ -275,16 +277,17 @@ AF_EXPORT int afm_sigattn_prefill_mfma(
     float scale, int ntiles, int H, int G, int dk, int dv, int page, int maxp,
     void* stream) {
   if (ntiles == 0) return 0;
-  if (G <= 0 || H % G || dk < 1 || dv < 1 || dk > 128 || dv > 128 || H > 16)
+  if (G <= 0 || H % G || dk < 1 || dv < 1 || dk > 128 || dv > 128 || H > 32)
     return 9003;
   if (RB > 0 && (!rel || !bucket_tab)) return 9003;
   const bool vec = (dk % 8 == 0) && (dv % 8 == 0) &&
                    ((uintptr_t)q % 16 == 0) && ((uintptr_t)kc % 16 == 0) &&
                    ((uintptr_t)vc % 16 == 0);
   const int hpw = H <= 4 ? 1 : H <= 8 ? 2 : 4;
+  const int nwv = (H + hpw - 1) / hpw;      // waves per workgroup, <= 8
   const int rep = H / G;
   int ngw = 1;
-  for (int w = 0; w < 4; ++w) {
+  for (int w = 0; w < nwv; ++w) {
     const int h0 = w * hpw, nh = H - h0 < hpw ? H - h0 : hpw;
     if (nh > 0) {
       const int n = (h0 + nh - 1) / rep - h0 / rep + 1;
@@ -294,7 +297,8 @@ AF_EXPORT int afm_sigattn_prefill_mfma(
   const bool small = dk <= 64 && dv <= 64;
   const int dvt = small ? 4 : 8;
   const size_t sm = (size_t)H * 2 * 64 * 16 +
-                    (size_t)4 * ngw * dvt * 16 * VS * 2 + 4 * 16 * VS * 2 +
+                    (size_t)nwv * ngw * dvt * 16 * VS * 2 +
+                    (size_t)nwv * 16 * VS * 2 +
                     (size_t)RB * H * 4 + (size_t)n_tab * 4 + 16;
   if (sm > 160 * 1024) return 9004;
   hipStream_t s = (hipStream_t)stream;
@@ -306,7 +310,7 @@ AF_EXPORT int afm_sigattn_prefill_mfma(
           hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm);               \
       if (e != hipSuccess) return (int)e;                                     \
     }                                                                         \
-    kern<<<ntiles, 256, sm, s>>>((u16*)out, (const u16*)q, (const u16*)kc,    \
+    kern<<<ntiles, 64 * nwv, sm, s>>>((u16*)out, (const u16*)q, (const u16*)kc,    \
         (const u16*)vc, (const i32*)bt, (const i32*)cu, (const i32*)q_start,  \
         (const i32*)tile_seq, (const i32*)tile_q0, (const float*)rel,         \
         (const i32*)bucket_tab, n_tab, RB, (const float*)talk,                \

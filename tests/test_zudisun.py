@@ -316,7 +316,9 @@ def _attn_run(m, P, h, v_first, device, dtype, portions, page=8):
                                    (1, 1, 8, 8, 2, 4, 3),
                                    (9, 3, 6, 10, 9, 31.5, 7),
                                    (6, 6, 24, 40, 12, 50, 1),
-                                   (20, 2, 8, 8, 16, 64, 1000)])
+                                   (20, 2, 8, 8, 16, 64, 1000),
+                                   (32, 8, 16, 24, 6, 33, 5),
+                                   (12, 4, 8, 8, 4, 9, 2)])
 def test_sigmoid_attention_alone(device, dtype, shape):
     H, G, dk, dv, rows, dmax, every = shape
     m, P, h, v_first = _attn_case(H, G, dk, dv, rows, dmax, every, dtype)
