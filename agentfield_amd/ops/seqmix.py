@@ -725,9 +725,12 @@ def distance_buckets(rows: int, dmax: float) -> torch.Tensor:
         if n < half:
             out.append(n)
             continue
+        if dmax <= half or half == 0:      # no logarithmic range at all
+            out.append(rows - 1)
+            continue
         v = math.log(n / half) / math.log(dmax / half) * (rows - half)
         out.append(min(rows - 1, half + int(math.floor(v + 1e-9))))
-    return torch.tensor(out, dtype=torch.int32)
+    return torch.tensor(out or [rows - 1], dtype=torch.int32)
 
 
 def qk_unit_cache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
