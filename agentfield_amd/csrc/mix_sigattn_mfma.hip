@@ -137,12 +137,13 @@ __global__ void __launch_bounds__(MAXT) sigattn_prefill_mfma_kernel(
   int pgk[2], pgv[2];
   pages_of(0, pgk, pgv);
 
-  // With the whole register file to a wave (MAXT = 256) the K fragments and
-  // the raw V rows of the NEXT tile, for the first PFG groups of the wave,
+  // Where registers allow (the whole file to a wave, or few heads per wave)
+  // the K fragments and the raw V rows of the NEXT tile, for the first PFG
+  // groups of the wave,
   // are fetched into registers while the current tile is mixed and
   // multiplied, so a tile starts with its operands already on chip.
-  constexpr bool PF = MAXT == 256;
-  constexpr int PFG = 2;
+  constexpr bool PF = MAXT == 256 || HPW <= 2;
+  constexpr int PFG = HPW <= 2 ? 1 : 2;
   constexpr int VIT = DVT / 2;             // V staging iterations per group
   s16x8 kpf[PF ? PFG : 1][2][DKC];
   s16x8 vpf[PF ? PFG : 1][VIT][2];
@@ -399,7 +400,8 @@ AF_EXPORT int afm_sigattn_prefill_mfma(
   const bool vec = (dk % 8 == 0) && (dv % 8 == 0) &&
                    ((uintptr_t)q % 16 == 0) && ((uintptr_t)kc % 16 == 0) &&
                    ((uintptr_t)vc % 16 == 0);
-  const int hpw = H <= 4 ? 1 : H <= 8 ? 2 : 4;
+  // up to eight waves: two waves per SIMD hide each other's LDS and MFMA waits
+  const int hpw = H <= 8 ? 1 : H <= 16 ? 2 : 4;
   const int nwv = (H + hpw - 1) / hpw;      // waves per workgroup, <= 8
   const int rep = H / G;
   int ngw = 1;
